@@ -1,0 +1,139 @@
+/*
+ * gmlp.h — C ABI of libgmlp.so: gated-MLP forward/backward kernels for AMD Instinct MI355X (gfx950).
+ *
+ * The library is the device half of a drop-in for the operator layer of matteobonotto/triton-gated-mlp.
+ * Every entry point below names the reference interface it stands behind (paths relative to the
+ * reference repository root).  The reference launches Triton JIT kernels from Python; here the same
+ * host wrappers load this library with ctypes and pass raw device pointers.
+ *
+ * Conventions
+ *   - All matrices are dense, row-major, contiguous, on the current HIP device, 16-byte aligned.
+ *   - M = tokens (rows of x), K = hidden_size, N = intermediate_size.
+ *     W_gate, W_up are [N,K]; W_down is [K,N]  (torch.nn.Linear [out,in] layout).
+ *   - dtype: GMLP_F16 or GMLP_BF16 storage; accumulation and epilogue arithmetic are fp32.
+ *   - Every call only ENQUEUES work on `stream` (a hipStream_t; NULL = default stream) and returns.
+ *     The library never allocates, frees or keeps device memory; the caller owns every buffer,
+ *     including workspaces (sizes from gmlp_workspace_bytes).
+ *   - Return value: 0 on success, a negative GMLP_E* code otherwise; nothing is launched on error.
+ *     gmlp_last_error() returns a thread-local message for the last failing call on this thread.
+ *   - Dropout: keep(m,n) = philox4x32_10(counter = {lo32(e/4), hi32(e/4), lo32(offset), hi32(offset)},
+ *     key = {lo32(seed), hi32(seed)})[e%4] >= floor(p * 2^32), with e = m*N + n; kept values are
+ *     scaled by 1/(1-p).  p == 0 disables dropout (the generator is not evaluated).
+ */
+#ifndef GMLP_H_
+#define GMLP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GMLP_ABI_VERSION 1
+
+enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1 };
+
+enum gmlp_status {
+  GMLP_OK = 0,
+  GMLP_EINVAL = -1, /* null pointer, bad dtype, bad dropout probability */
+  GMLP_ESHAPE = -2, /* shape not supported (see each entry point) */
+  GMLP_EALIGN = -3, /* pointer not 16-byte aligned */
+  GMLP_EHIP = -4    /* HIP runtime reported an error at launch */
+};
+
+enum gmlp_op { GMLP_OP_DECODE_FWD = 0, GMLP_OP_COLSUM = 1 };
+
+int gmlp_abi_version(void);
+const char* gmlp_last_error(void);
+
+/* Workspace bytes the caller must provide for `op` at the given problem size (0 if none). */
+size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
+
+/*
+ * Hidden-state forward:  G = x·W_gateᵀ + b_gate,  U = x·W_upᵀ + b_up,
+ *                        H = dropout(silu(G) ⊙ U).
+ * Replaces mlp_hidden_states_fwd + _fwd_kernel (src/triton_gated_mlp/ops/fwd.py:198-279, :72-166);
+ * math of EagerGatedMLP.forward (src/triton_gated_mlp/gated_mlp.py:96) and eager_fwd (:105-128).
+ * b_gate, b_up, g_save, u_save, mask_out may be NULL.  g_save/u_save [M,N] receive G and U
+ * (activations kept for the backward pass).  mask_out [M,N] uint8 receives the keep mask.
+ * Requires K % 8 == 0, N % 8 == 0, M >= 1.
+ */
+int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
+                    const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
+                    int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                    uint64_t offset, void* stream);
+
+/*
+ * Linear layer forward: out[M,C] = a[M,R]·w[C,R]ᵀ + bias[C]   (bias may be NULL).
+ * Replaces the nn.Linear down_proj call (src/triton_gated_mlp/gated_mlp.py:236), which the
+ * reference leaves to the vendor BLAS.  Requires R % 8 == 0, C % 8 == 0.
+ */
+int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, int64_t M, int64_t R,
+                    int64_t C, int dtype, void* stream);
+
+/*
+ * Backward through down_proj, dropout and the gating product in one GEMM:
+ *   dH = dY·W_down ; dA = dH ⊙ keep/(1-p) ; dU = dA ⊙ silu(G) ; dG = dA ⊙ U ⊙ silu'(G).
+ * Replaces the autograd backward of down_proj plus _compute_quantities_for_bwd
+ * (src/triton_gated_mlp/ops/bwd.py:89-211; closed form in gated_mlp.py:131-144).  g, u are the
+ * tensors written by gmlp_gateup_fwd (g_save, u_save).  dg, du are [M,N].
+ */
+int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
+                int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                uint64_t offset, void* stream);
+
+/*
+ * Element-wise gating backward for callers that already hold dH (the reference's operator-level
+ * backward receives grad_output = dH):  dU = dA ⊙ silu(G), dG = dA ⊙ U ⊙ silu'(G), dA as above.
+ * Replaces the epilogue of _compute_quantities_for_bwd (src/triton_gated_mlp/ops/bwd.py:196-211).
+ */
+int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t M,
+                    int64_t N, int dtype, float dropout_p, uint64_t seed, uint64_t offset,
+                    void* stream);
+
+/*
+ * dX = dG·W_gate + dU·W_up   (one GEMM over the concatenated reduction of length 2N).
+ * Replaces _compute_dx (src/triton_gated_mlp/ops/bwd.py:242-322; gated_mlp.py:147-149).
+ */
+int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* w_up, void* dx,
+                int64_t M, int64_t K, int64_t N, int dtype, void* stream);
+
+/*
+ * Weight gradient: dw[R,C] = lhs[Mred,R]ᵀ · rhs[Mred,C].
+ * Replaces _compute_dW_up_dW_gp (src/triton_gated_mlp/ops/bwd.py:386-463; gated_mlp.py:152-155)
+ * with (lhs,rhs) = (dG,x), (dU,x); and the autograd dW of down_proj with (lhs,rhs) = (dY,H).
+ * Requires R % 8 == 0, C % 8 == 0.
+ */
+int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_t R, int64_t C,
+                int dtype, void* stream);
+
+/*
+ * Bias gradient: out[C] = Σ_m a[m,C], fp32 accumulation in a fixed order (deterministic).
+ * workspace: gmlp_workspace_bytes(GMLP_OP_COLSUM, M, 0, C, dtype) bytes.
+ * The reference returns None for bias gradients (gated_mlp.py:200); EagerGatedMLP's autograd
+ * produces them, and this entry point supplies them.
+ */
+int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C, int dtype,
+                void* stream);
+
+/*
+ * Skinny-M forward of the whole MLP (decode): y = (silu(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
+ * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch is [M,N] in dtype;
+ * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
+ * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
+ * Requires K % 512 == 0 and N % 512 == 0.
+ */
+int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
+                    const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
+                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype,
+                    void* stream);
+
+/* Writes the dropout keep mask (1 = keep) for an [M,N] tensor; the test oracle of the generator. */
+int gmlp_dropout_mask(uint8_t* mask, int64_t M, int64_t N, float dropout_p, uint64_t seed,
+                      uint64_t offset, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GMLP_H_ */

@@ -1,0 +1,276 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on identical seeded inputs.
+
+Tolerance: rtol = atol = 2e-2 element-wise for fp16/bf16 storage with fp32 accumulation, against
+the oracle evaluated in fp32 on the same (already rounded) inputs.
+"""
+
+import contextlib
+
+import numpy as np
+import pytest
+import torch
+
+from cases import CFG2, CFG3, CFG4, CFG5, Case, make_inputs
+from oracle import eager as oracle
+from oracle import philox
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 2e-2
+
+
+def _dev():
+    assert torch.cuda.is_available(), "GPU tests need a visible AMD GPU"
+    return torch.device("cuda", 0)
+
+
+def _close(name, got, ref, rtol=RTOL, atol=ATOL):
+    got = got.detach().float().cpu()
+    ref = ref.detach().float().cpu()
+    assert got.shape == ref.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    err = (got - ref).abs()
+    bound = atol + rtol * ref.abs()
+    bad = err > bound
+    rel_fro = ((got - ref).norm() / ref.norm().clamp_min(1e-30)).item()
+    print(f"  {name}: max_abs_err={err.max().item():.3e} rel_fro={rel_fro:.3e}", flush=True)
+    assert not bad.any(), (
+        f"{name}: {int(bad.sum())} of {bad.numel()} elements outside rtol={rtol}, atol={atol}; "
+        f"max_abs_err={err.max().item():.4e}, rel_fro={rel_fro:.3e}"
+    )
+    assert rel_fro < 1e-2, f"{name}: relative Frobenius error {rel_fro:.3e}"
+
+
+def _oracle_inputs(t):
+    return {k: (None if v is None else v.float()) for k, v in t.items()}
+
+
+def _run_module_case(c: Case):
+    from triton_gated_mlp import FusedGatedMLP
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    print(f"case {c.name}: M={c.M} K={c.K} N={c.N} dtype={c.dtype} bias={c.bias} p={c.p}", flush=True)
+    t = make_inputs(c)
+    mlp = FusedGatedMLP(hidden_size=c.K, intermediate_size=c.N, bias=c.bias, dropout_p=c.p).to(dev).to(c.dtype)
+    with torch.no_grad():
+        mlp.gate_proj.weight.copy_(t["W_gate"])
+        mlp.up_proj.weight.copy_(t["W_up"])
+        mlp.down_proj.weight.copy_(t["W_down"])
+        if c.bias:
+            mlp.gate_proj.bias.copy_(t["b_gate"])
+            mlp.up_proj.bias.copy_(t["b_up"])
+            mlp.down_proj.bias.copy_(t["b_down"])
+    mlp.train(c.p > 0.0)
+    mlp.dropout_seed = c.dropout_seed
+    x = t["x"].to(dev).requires_grad_(c.backward)
+
+    with contextlib.nullcontext() if c.backward else torch.no_grad():
+        y = mlp(x)
+    keep = None
+    if c.p > 0.0:
+        seed, offset = mlp.last_dropout_state
+        keep_dev = ops_fwd.dropout_mask(c.M, c.N, c.p, seed, offset, device=dev)
+        keep_np = philox.keep_mask(c.M, c.N, c.p, seed, offset)
+        assert np.array_equal(keep_dev.cpu().numpy(), keep_np), "device keep mask differs from the NumPy Philox oracle"
+        keep = torch.from_numpy(keep_np)
+
+    o = _oracle_inputs(t)
+    if not c.backward:
+        ref = oracle.forward(o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], keep, c.p)
+        _close("Y", y, ref["Y"])
+        return
+    grads_in = [x, mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight]
+    names = ["dX", "dW_gate", "dW_up", "dW_down"]
+    if c.bias:
+        grads_in += [mlp.gate_proj.bias, mlp.up_proj.bias, mlp.down_proj.bias]
+        names += ["db_gate", "db_up", "db_down"]
+    grads = torch.autograd.grad(y, grads_in, grad_outputs=t["dY"].to(dev))
+    ref = oracle.backward(
+        o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], o["dY"], keep, c.p
+    )
+    _close("Y", y, ref["Y"])
+    for n, g in zip(names, grads):
+        # weight gradients sum M terms: scale the absolute tolerance with the magnitude of the result
+        scale = max(1.0, ref[n].abs().mean().item())
+        _close(n, g, ref[n], atol=ATOL * scale)
+
+
+def test_cfg2_fp16_forward_llama7b():
+    _run_module_case(CFG2)
+
+
+def test_cfg3_fp16_forward_backward_llama3_8b():
+    _run_module_case(CFG3)
+
+
+def test_cfg4_bf16_bias_dropout_forward_backward():
+    _run_module_case(CFG4)
+
+
+def test_cfg5_fp16_decode_forward():
+    _run_module_case(CFG5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize(
+    "M,K,N,bias,p",
+    [
+        (128, 256, 512, True, 0.0),  # the reference's module test shape (tests/test_gated_mlp_fwd.py:23-38)
+        (512, 256, 512, False, 0.0),  # 3-D input case B=16, M=32 (tests/test_gated_mlp_bwd.py:27-45)
+        (64, 256, 512, False, 0.0),  # B,M,N,K = 2,32,512,256 (tests/test_gated_mlp_bwd.py:97)
+        (200, 136, 264, True, 0.25),  # ragged: nothing a multiple of the tile
+        (1, 64, 128, True, 0.0),
+        (256, 512, 1024, True, 0.5),
+        (768, 1024, 2048, False, 0.0),
+    ],
+)
+def test_small_shapes_forward_backward(M, K, N, bias, p, dtype):
+    _run_module_case(Case(f"small_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=p, backward=True, seed=M + K + N))
+
+
+def test_three_dimensional_input_matches_flattened():
+    """[B, S, K] input gives the 2-D result on x.view(-1, K) (tests/test_gated_mlp_bwd.py:37-45)."""
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    torch.manual_seed(0)
+    mlp = FusedGatedMLP(256, 512, bias=False).to(dev).to(torch.float16)
+    x = torch.rand(16, 32, 256, device=dev, dtype=torch.float16)
+    y3 = mlp(x)
+    y2 = mlp(x.view(-1, 256))
+    assert y3.shape == x.shape
+    assert torch.equal(y3.view(-1, 256), y2)
+
+
+def test_operator_level_fwd_bwd_match_closed_form():
+    """mlp_hidden_states_fwd/bwd against the closed form (pattern of tests/test_gated_mlp_bwd.py:89-129)."""
+    from triton_gated_mlp import mlp_hidden_states_bwd, mlp_hidden_states_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(7)
+    BM, N, K = 64, 512, 256
+    x = torch.rand(BM, K, generator=g).half()
+    W_up = (torch.rand(N, K, generator=g) / 8).half()
+    W_gp = (torch.rand(N, K, generator=g) / 8).half()
+    dH = torch.rand(BM, N, generator=g).half()
+    h = mlp_hidden_states_fwd(x.to(dev), W_up.to(dev), None, W_gp.to(dev), None, "silu", 0.0)
+    ref = oracle.hidden_forward(x.float(), W_gp.float(), None, W_up.float(), None)
+    _close("hidden", h, ref["H"])
+    dx, dW_up, dW_gp = mlp_hidden_states_bwd(x.to(dev), W_up.to(dev), W_gp.to(dev), dH.to(dev))
+    hb = oracle.hidden_backward(dH.float(), ref["G"], ref["U"])
+    _close("dx", dx, hb["dU"] @ W_up.float() + hb["dG"] @ W_gp.float(), atol=ATOL * 4)
+    _close("dW_up", dW_up, hb["dU"].T @ x.float(), atol=ATOL * 4)
+    _close("dW_gp", dW_gp, hb["dG"].T @ x.float(), atol=ATOL * 4)
+
+
+def test_autograd_function_reference_signature():
+    """FusedGatedMLPFunction.apply(x, W_up, b_up, W_gp, b_gp) with biases and bias gradients."""
+    from triton_gated_mlp import FusedGatedMLPFunction
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(11)
+    M, K, N = 96, 128, 256
+    mk = lambda *s: torch.randn(*s, generator=g).mul(0.1).half()
+    x, W_up, b_up, W_gp, b_gp, dH = mk(M, K), mk(N, K), mk(N), mk(N, K), mk(N), mk(M, N)
+    args = [a.to(dev).requires_grad_(True) for a in (x, W_up, b_up, W_gp, b_gp)]
+    h = FusedGatedMLPFunction.apply(*args)
+    grads = torch.autograd.grad(h, args, grad_outputs=dH.to(dev))
+    ref_in = [a.float().requires_grad_(True) for a in (x, W_up, b_up, W_gp, b_gp)]
+    ref = oracle.hidden_forward(ref_in[0], ref_in[3], ref_in[4], ref_in[1], ref_in[2])["H"]
+    ref_grads = torch.autograd.grad(ref, ref_in, grad_outputs=dH.float())
+    _close("hidden", h, ref)
+    for n, a, b in zip(("dx", "dW_up", "db_up", "dW_gp", "db_gp"), grads, ref_grads):
+        _close(n, a, b)
+
+
+def test_eval_mode_ignores_dropout_and_is_deterministic():
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    torch.manual_seed(3)
+    mlp = FusedGatedMLP(256, 512, bias=True, dropout_p=0.5).to(dev).to(torch.bfloat16)
+    x = torch.randn(64, 256, device=dev, dtype=torch.bfloat16)
+    mlp.eval()
+    y0, y1 = mlp(x), mlp(x)
+    assert torch.equal(y0, y1)
+    mlp.train()
+    mlp.dropout_seed = 5
+    a = mlp(x)
+    mlp._dropout_calls = 0
+    b = mlp(x)
+    assert torch.equal(a, b), "same seed and offset must give the same mask"
+    assert not torch.equal(a, y0)
+
+
+def test_dropout_mask_matches_numpy_philox_and_rate():
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    for (M, N, p, seed, off) in [(64, 128, 0.1, 1234, 0), (33, 72, 0.5, 2**40 + 17, 3), (1024, 2048, 0.25, 99, 2**33)]:
+        got = ops_fwd.dropout_mask(M, N, p, seed, off, device=dev).cpu().numpy()
+        ref = philox.keep_mask(M, N, p, seed, off)
+        assert np.array_equal(got, ref)
+        rate = got.mean()
+        sigma = (p * (1 - p) / (M * N)) ** 0.5
+        assert abs(rate - (1 - p)) < 5 * sigma + 1e-9
+
+
+def test_forward_mask_output_equals_standalone_mask():
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(5)
+    M, K, N = 300, 128, 520
+    x = torch.randn(M, K, generator=g).half().to(dev)
+    Wg = (0.05 * torch.randn(N, K, generator=g)).half().to(dev)
+    Wu = (0.05 * torch.randn(N, K, generator=g)).half().to(dev)
+    hs = ops_fwd.gateup_fwd(x, Wg, None, Wu, None, 0.3, seed=77, offset=1, save_activations=True, return_mask=True)
+    ref = philox.keep_mask(M, N, 0.3, 77, 1)
+    assert np.array_equal(hs.mask.cpu().numpy(), ref)
+    o = oracle.hidden_forward(x.float().cpu(), Wg.float().cpu(), None, Wu.float().cpu(), None, torch.from_numpy(ref), 0.3)
+    _close("H", hs.hidden, o["H"])
+    _close("G", hs.gate, o["G"])
+    _close("U", hs.up, o["U"])
+
+
+def test_full_size_properties_cfg3_linearity_and_zero():
+    """Size-independent checks at the headline shape: x = 0 gives Y = 0 (no bias), and the down
+    projection is linear in H (Y(2H) = 2Y(H))."""
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    c = CFG3
+    g = torch.Generator(device="cpu").manual_seed(1)
+    Wd = (0.02 * torch.randn(c.K, c.N, generator=g)).half().to(dev)
+    H = torch.randn(c.M, c.N, generator=g).half().to(dev)
+    y1 = ops_fwd.linear_fwd(H, Wd)
+    y2 = ops_fwd.linear_fwd(H * 2, Wd)
+    assert torch.allclose(y2.float(), 2 * y1.float(), rtol=2e-3, atol=2e-3)
+    Wg = (0.02 * torch.randn(c.N, c.K, generator=g)).half().to(dev)
+    z = ops_fwd.gateup_fwd(torch.zeros(c.M, c.K, dtype=torch.float16, device=dev), Wg, None, Wg, None)
+    assert not z.hidden.any()
+
+
+def test_decode_matches_general_path():
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(2)
+    for M, K, N, bias in [(16, 1024, 2048, True), (3, 256, 512, False), (1, 4096, 11008, True)]:
+        x = torch.randn(M, K, generator=g).half().to(dev)
+        Wg = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
+        Wu = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
+        Wd = (0.02 * torch.randn(K, N, generator=g)).half().to(dev)
+        bg = bu = bd = None
+        if bias:
+            bg = (0.01 * torch.randn(N, generator=g)).half().to(dev)
+            bu = (0.01 * torch.randn(N, generator=g)).half().to(dev)
+            bd = (0.01 * torch.randn(K, generator=g)).half().to(dev)
+        y = ops_fwd.decode_fwd(x, Wg, bg, Wu, bu, Wd, bd)
+        f = lambda t: None if t is None else t.float().cpu()
+        ref = oracle.forward(f(x), f(Wg), f(bg), f(Wu), f(bu), f(Wd), f(bd))
+        _close(f"decode Y M={M}", y, ref["Y"])
+        h = ops_fwd.gateup_fwd(x, Wg, bg, Wu, bu).hidden
+        y_general = ops_fwd.linear_fwd(h, Wd, bd)
+        _close(f"general Y M={M}", y_general, ref["Y"])

@@ -1,0 +1,326 @@
+// extern "C" entry points of libgmlp.so (declared in include/gmlp.h): argument validation,
+// tile-class selection and kernel launches.  All validation happens before the first HIP call,
+// so the error paths can be exercised on a machine without a GPU.
+#include "gmlp.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+
+#include "launch.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define GMLP_REQUIRE_PTR(p)                                                         \
+  if ((p) == nullptr) return fail(GMLP_EINVAL, "%s: argument '%s' is NULL", __func__, #p)
+#define GMLP_REQUIRE_ALIGNED(p)                                                     \
+  if ((p) != nullptr && !aligned16(p))                                              \
+  return fail(GMLP_EALIGN, "%s: argument '%s' is not 16-byte aligned", __func__, #p)
+#define GMLP_REQUIRE_DTYPE(d)                                                       \
+  if ((d) != GMLP_F16 && (d) != GMLP_BF16)                                          \
+  return fail(GMLP_EINVAL, "%s: dtype %d is not GMLP_F16/GMLP_BF16", __func__, (int)(d))
+
+const int64_t kMaxDim = (int64_t)1 << 30;
+
+int check_dims(const char* fn, int64_t M, int64_t K, int64_t N) {
+  if (M < 1 || K < 1 || N < 1) return fail(GMLP_ESHAPE, "%s: M, K, N must be >= 1 (got %lld, %lld, %lld)", fn,
+                                           (long long)M, (long long)K, (long long)N);
+  if (M > kMaxDim || K > kMaxDim || N > kMaxDim || M * N >= ((int64_t)1 << 40) ||
+      M * K >= ((int64_t)1 << 40))
+    return fail(GMLP_ESHAPE, "%s: dimension too large", fn);
+  return 0;
+}
+
+int check_mult8(const char* fn, const char* name, int64_t v) {
+  if (v % 8 != 0)
+    return fail(GMLP_ESHAPE, "%s: %s = %lld must be a multiple of 8 (16-byte rows)", fn, name, (long long)v);
+  return 0;
+}
+
+int make_dropout(const char* fn, float p, uint64_t seed, uint64_t offset, gmlp::DropoutParams* d) {
+  if (!(p >= 0.0f) || !(p < 1.0f))
+    return fail(GMLP_EINVAL, "%s: dropout_p = %g must satisfy 0 <= p < 1", fn, (double)p);
+  d->enabled = p > 0.0f ? 1 : 0;
+  double t = std::floor((double)p * 4294967296.0);
+  d->threshold = t >= 4294967295.0 ? 4294967295u : (uint32_t)t;
+  d->scale = 1.0f / (1.0f - p);
+  d->seed_lo = (uint32_t)seed;
+  d->seed_hi = (uint32_t)(seed >> 32);
+  d->off_lo = (uint32_t)offset;
+  d->off_hi = (uint32_t)(offset >> 32);
+  return 0;
+}
+
+int hip_result(const char* fn, hipError_t e) {
+  if (e == hipSuccess) return GMLP_OK;
+  return fail(GMLP_EHIP, "%s: HIP error %d (%s)", fn, (int)e, hipGetErrorString(e));
+}
+
+// LARGE tiles need whole 256 x bn_large tiles, a reduction that is a multiple of 64, and enough
+// tiles to occupy the chip; everything else runs on the predicated MEDIUM class.
+int pick_tile(int64_t rows, int64_t cols, int64_t red, int bn_large) {
+  if (rows % 256 == 0 && cols % bn_large == 0 && red % 64 == 0 &&
+      (rows / 256) * (cols / bn_large) >= 192)
+    return gmlp::TILE_LARGE;
+  return gmlp::TILE_MEDIUM;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gmlp_abi_version(void) { return GMLP_ABI_VERSION; }
+const char* gmlp_last_error(void) { return g_err; }
+
+size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {
+  (void)K;
+  (void)dtype;
+  if (op == GMLP_OP_COLSUM && M >= 1 && N >= 1) return gmlp::colsum_workspace_bytes(M, N);
+  return 0;
+}
+
+int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
+                    const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
+                    int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                    uint64_t offset, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(x); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up); GMLP_REQUIRE_PTR(h);
+  GMLP_REQUIRE_DTYPE(dtype);
+  DropoutParams d;
+  if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
+  if (int rc = check_dims(__func__, M, K, N)) return rc;
+  if (int rc = check_mult8(__func__, "K", K)) return rc;
+  if (int rc = check_mult8(__func__, "N", N)) return rc;
+  GMLP_REQUIRE_ALIGNED(x); GMLP_REQUIRE_ALIGNED(w_gate); GMLP_REQUIRE_ALIGNED(w_up);
+  GMLP_REQUIRE_ALIGNED(b_gate); GMLP_REQUIRE_ALIGNED(b_up); GMLP_REQUIRE_ALIGNED(h);
+  GMLP_REQUIRE_ALIGNED(g_save); GMLP_REQUIRE_ALIGNED(u_save); GMLP_REQUIRE_ALIGNED(mask_out);
+
+  GemmArgs ga = {};
+  ga.A[0] = x; ga.A[1] = x; ga.B[0] = w_gate; ga.B[1] = w_up;
+  ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
+  ga.nseg = 1; ga.group_m = 8;
+  int tc = pick_tile(M, N, K, 128);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    EpiGateUp<f16>::Args ea = {(f16*)h, (f16*)g_save, (f16*)u_save, mask_out, (const f16*)b_gate,
+                               (const f16*)b_up, (int)N, d};
+    e = launch_gateup<f16>(tc, ga, ea, s);
+  } else {
+    EpiGateUp<bf16>::Args ea = {(bf16*)h, (bf16*)g_save, (bf16*)u_save, mask_out,
+                                (const bf16*)b_gate, (const bf16*)b_up, (int)N, d};
+    e = launch_gateup<bf16>(tc, ga, ea, s);
+  }
+  return hip_result(__func__, e);
+}
+
+int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, int64_t M, int64_t R,
+                    int64_t C, int dtype, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(w); GMLP_REQUIRE_PTR(out);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, M, R, C)) return rc;
+  if (int rc = check_mult8(__func__, "R", R)) return rc;
+  if (int rc = check_mult8(__func__, "C", C)) return rc;
+  GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(w); GMLP_REQUIRE_ALIGNED(bias);
+  GMLP_REQUIRE_ALIGNED(out);
+
+  GemmArgs ga = {};
+  ga.A[0] = a; ga.A[1] = a; ga.B[0] = w; ga.B[1] = w;
+  ga.M = (int)M; ga.N = (int)C; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
+  ga.nseg = 1; ga.group_m = 8;
+  int tc = pick_tile(M, C, R, 256);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    EpiStore<f16>::Args ea = {(f16*)out, (const f16*)bias, (int)C};
+    e = launch_linear<f16>(tc, ga, ea, s);
+  } else {
+    EpiStore<bf16>::Args ea = {(bf16*)out, (const bf16*)bias, (int)C};
+    e = launch_linear<bf16>(tc, ga, ea, s);
+  }
+  return hip_result(__func__, e);
+}
+
+int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
+                int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                uint64_t offset, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(dy); GMLP_REQUIRE_PTR(w_down); GMLP_REQUIRE_PTR(g); GMLP_REQUIRE_PTR(u);
+  GMLP_REQUIRE_PTR(dg); GMLP_REQUIRE_PTR(du);
+  GMLP_REQUIRE_DTYPE(dtype);
+  DropoutParams d;
+  if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
+  if (int rc = check_dims(__func__, M, K, N)) return rc;
+  if (int rc = check_mult8(__func__, "K", K)) return rc;
+  if (int rc = check_mult8(__func__, "N", N)) return rc;
+  GMLP_REQUIRE_ALIGNED(dy); GMLP_REQUIRE_ALIGNED(w_down); GMLP_REQUIRE_ALIGNED(g);
+  GMLP_REQUIRE_ALIGNED(u); GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du);
+
+  // dH[M,N] = dY[M,K] · W_down[K,N]: reduction over K; B is reduction-strided ([K,N] row-major).
+  GemmArgs ga = {};
+  ga.A[0] = dy; ga.A[1] = dy; ga.B[0] = w_down; ga.B[1] = w_down;
+  ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
+  ga.nseg = 1; ga.group_m = 8;
+  int tc = pick_tile(M, N, K, 256);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    EpiDh<f16>::Args ea = {(const f16*)g, (const f16*)u, (f16*)dg, (f16*)du, (int)N, d};
+    e = launch_dh<f16>(tc, ga, ea, s);
+  } else {
+    EpiDh<bf16>::Args ea = {(const bf16*)g, (const bf16*)u, (bf16*)dg, (bf16*)du, (int)N, d};
+    e = launch_dh<bf16>(tc, ga, ea, s);
+  }
+  return hip_result(__func__, e);
+}
+
+int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t M,
+                    int64_t N, int dtype, float dropout_p, uint64_t seed, uint64_t offset,
+                    void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(dh); GMLP_REQUIRE_PTR(g); GMLP_REQUIRE_PTR(u); GMLP_REQUIRE_PTR(dg);
+  GMLP_REQUIRE_PTR(du);
+  GMLP_REQUIRE_DTYPE(dtype);
+  DropoutParams d;
+  if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
+  if (int rc = check_dims(__func__, M, 8, N)) return rc;
+  if (int rc = check_mult8(__func__, "N", N)) return rc;
+  GMLP_REQUIRE_ALIGNED(dh); GMLP_REQUIRE_ALIGNED(g); GMLP_REQUIRE_ALIGNED(u);
+  GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = dtype == GMLP_F16
+                     ? launch_gating_bwd<f16>((const f16*)dh, (const f16*)g, (const f16*)u, (f16*)dg,
+                                              (f16*)du, M, N, d, s)
+                     : launch_gating_bwd<bf16>((const bf16*)dh, (const bf16*)g, (const bf16*)u,
+                                               (bf16*)dg, (bf16*)du, M, N, d, s);
+  return hip_result(__func__, e);
+}
+
+int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* w_up, void* dx,
+                int64_t M, int64_t K, int64_t N, int dtype, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(dg); GMLP_REQUIRE_PTR(du); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up);
+  GMLP_REQUIRE_PTR(dx);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, M, K, N)) return rc;
+  if (int rc = check_mult8(__func__, "K", K)) return rc;
+  if (int rc = check_mult8(__func__, "N", N)) return rc;
+  GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du); GMLP_REQUIRE_ALIGNED(w_gate);
+  GMLP_REQUIRE_ALIGNED(w_up); GMLP_REQUIRE_ALIGNED(dx);
+
+  // dX[M,K] = dG[M,N]·W_gate[N,K] + dU[M,N]·W_up[N,K]: two reduction segments of length N.
+  GemmArgs ga = {};
+  ga.A[0] = dg; ga.A[1] = du; ga.B[0] = w_gate; ga.B[1] = w_up;
+  ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
+  ga.nseg = 2; ga.group_m = 8;
+  int tc = pick_tile(M, K, N, 256);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    EpiStore<f16>::Args ea = {(f16*)dx, nullptr, (int)K};
+    e = launch_dx<f16>(tc, ga, ea, s);
+  } else {
+    EpiStore<bf16>::Args ea = {(bf16*)dx, nullptr, (int)K};
+    e = launch_dx<bf16>(tc, ga, ea, s);
+  }
+  return hip_result(__func__, e);
+}
+
+int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_t R, int64_t C,
+                int dtype, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(lhs); GMLP_REQUIRE_PTR(rhs); GMLP_REQUIRE_PTR(dw);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, Mred, R, C)) return rc;
+  if (int rc = check_mult8(__func__, "R", R)) return rc;
+  if (int rc = check_mult8(__func__, "C", C)) return rc;
+  GMLP_REQUIRE_ALIGNED(lhs); GMLP_REQUIRE_ALIGNED(rhs); GMLP_REQUIRE_ALIGNED(dw);
+
+  // dW[R,C] = lhs[Mred,R]ᵀ · rhs[Mred,C]: both operands reduction-strided.
+  GemmArgs ga = {};
+  ga.A[0] = lhs; ga.A[1] = lhs; ga.B[0] = rhs; ga.B[1] = rhs;
+  ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
+  ga.nseg = 1; ga.group_m = 8;
+  int tc = pick_tile(R, C, Mred, 256);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    EpiStore<f16>::Args ea = {(f16*)dw, nullptr, (int)C};
+    e = launch_dw<f16>(tc, ga, ea, s);
+  } else {
+    EpiStore<bf16>::Args ea = {(bf16*)dw, nullptr, (int)C};
+    e = launch_dw<bf16>(tc, ga, ea, s);
+  }
+  return hip_result(__func__, e);
+}
+
+int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C, int dtype,
+                void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(out); GMLP_REQUIRE_PTR(workspace);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, M, 8, C)) return rc;
+  if (int rc = check_mult8(__func__, "C", C)) return rc;
+  GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(out); GMLP_REQUIRE_ALIGNED(workspace);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = dtype == GMLP_F16
+                     ? launch_colsum<f16>((const f16*)a, (f16*)out, (float*)workspace, M, C, s)
+                     : launch_colsum<bf16>((const bf16*)a, (bf16*)out, (float*)workspace, M, C, s);
+  return hip_result(__func__, e);
+}
+
+int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
+                    const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
+                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype,
+                    void* stream) {
+  using namespace gmlp;
+  (void)workspace;
+  GMLP_REQUIRE_PTR(x); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up); GMLP_REQUIRE_PTR(w_down);
+  GMLP_REQUIRE_PTR(h_scratch); GMLP_REQUIRE_PTR(y);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, M, K, N)) return rc;
+  if (M > 16) return fail(GMLP_ESHAPE, "%s: M = %lld exceeds the skinny-M limit of 16", __func__, (long long)M);
+  if (K % 32 != 0) return fail(GMLP_ESHAPE, "%s: K = %lld must be a multiple of 32", __func__, (long long)K);
+  if (N % 256 != 0) return fail(GMLP_ESHAPE, "%s: N = %lld must be a multiple of 256", __func__, (long long)N);
+  GMLP_REQUIRE_ALIGNED(x); GMLP_REQUIRE_ALIGNED(w_gate); GMLP_REQUIRE_ALIGNED(w_up);
+  GMLP_REQUIRE_ALIGNED(w_down); GMLP_REQUIRE_ALIGNED(b_gate); GMLP_REQUIRE_ALIGNED(b_up);
+  GMLP_REQUIRE_ALIGNED(b_down); GMLP_REQUIRE_ALIGNED(h_scratch); GMLP_REQUIRE_ALIGNED(y);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e =
+      dtype == GMLP_F16
+          ? launch_decode<f16>((const f16*)x, (const f16*)w_gate, (const f16*)w_up, (const f16*)w_down,
+                               (const f16*)b_gate, (const f16*)b_up, (const f16*)b_down,
+                               (f16*)h_scratch, (f16*)y, (int)M, (int)K, (int)N, s)
+          : launch_decode<bf16>((const bf16*)x, (const bf16*)w_gate, (const bf16*)w_up,
+                                (const bf16*)w_down, (const bf16*)b_gate, (const bf16*)b_up,
+                                (const bf16*)b_down, (bf16*)h_scratch, (bf16*)y, (int)M, (int)K,
+                                (int)N, s);
+  return hip_result(__func__, e);
+}
+
+int gmlp_dropout_mask(uint8_t* mask, int64_t M, int64_t N, float dropout_p, uint64_t seed,
+                      uint64_t offset, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(mask);
+  DropoutParams d;
+  if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
+  if (int rc = check_dims(__func__, M, 8, N)) return rc;
+  if (int rc = check_mult8(__func__, "N", N)) return rc;
+  GMLP_REQUIRE_ALIGNED(mask);
+  return hip_result(__func__, launch_dropout_mask(mask, M, N, d, (hipStream_t)stream));
+}
+
+}  // extern "C"

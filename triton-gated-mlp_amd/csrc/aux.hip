@@ -1,0 +1,99 @@
+// HBM-bound helper kernels: element-wise gating backward, deterministic column sums (bias
+// gradients) and the stand-alone dropout keep-mask generator.
+#include "launch.hpp"
+
+namespace gmlp {
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    gating_bwd_kernel(const T* __restrict__ dh, const T* __restrict__ g, const T* __restrict__ u,
+                      T* __restrict__ dg, T* __restrict__ du, size_t n4, DropoutParams d) {
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    size_t e = i * 4;
+    gating_bwd4<T>(d, e, load4<T>(dh + e), g, u, dg, du);
+  }
+}
+
+template <typename T>
+hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
+                             const DropoutParams& d, hipStream_t s) {
+  size_t n4 = (size_t)M * N / 4;
+  if (n4 == 0) return hipSuccess;
+  size_t blocks = (n4 + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(gating_bwd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, dh, g, u, dg, du,
+                     n4, d);
+  return hipGetLastError();
+}
+template hipError_t launch_gating_bwd<f16>(const f16*, const f16*, const f16*, f16*, f16*, int64_t,
+                                           int64_t, const DropoutParams&, hipStream_t);
+template hipError_t launch_gating_bwd<bf16>(const bf16*, const bf16*, const bf16*, bf16*, bf16*,
+                                            int64_t, int64_t, const DropoutParams&, hipStream_t);
+
+// Column sums in two fixed-order stages: COLSUM_SPLITS row ranges -> fp32 partials -> total.
+constexpr int COLSUM_SPLITS = 64;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    colsum_partial_kernel(const T* __restrict__ a, float* __restrict__ ws, int64_t M, int64_t C) {
+  int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  int64_t rows = (M + COLSUM_SPLITS - 1) / COLSUM_SPLITS;
+  int64_t r0 = blockIdx.y * rows, r1 = r0 + rows < M ? r0 + rows : M;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t r = r0; r < r1; ++r) s += load4<T>(a + r * C + c);
+  *(f32x4*)(ws + (int64_t)blockIdx.y * C + c) = s;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    colsum_final_kernel(const float* __restrict__ ws, T* __restrict__ out, int64_t C) {
+  int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < COLSUM_SPLITS; ++i) s += *(const f32x4*)(ws + (int64_t)i * C + c);
+  store4<T>(out + c, s);
+}
+
+size_t colsum_workspace_bytes(int64_t, int64_t C) { return (size_t)COLSUM_SPLITS * C * sizeof(float); }
+
+template <typename T>
+hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s) {
+  unsigned bx = (unsigned)((C / 4 + 255) / 256);
+  hipLaunchKernelGGL(colsum_partial_kernel<T>, dim3(bx, COLSUM_SPLITS), dim3(256), 0, s, a, ws, M, C);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(colsum_final_kernel<T>, dim3(bx), dim3(256), 0, s, ws, out, C);
+  return hipGetLastError();
+}
+template hipError_t launch_colsum<f16>(const f16*, f16*, float*, int64_t, int64_t, hipStream_t);
+template hipError_t launch_colsum<bf16>(const bf16*, bf16*, float*, int64_t, int64_t, hipStream_t);
+
+__global__ void __launch_bounds__(256)
+    dropout_mask_kernel(uint8_t* __restrict__ mask, size_t n4, DropoutParams d) {
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    bool keep[4];
+    uint32_t packed = 0x01010101u;
+    if (d.enabled) {
+      dropout_keep4(d, i, keep);
+      packed = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) packed |= (keep[r] ? 1u : 0u) << (8 * r);
+    }
+    *(uint32_t*)(mask + i * 4) = packed;
+  }
+}
+
+hipError_t launch_dropout_mask(uint8_t* mask, int64_t M, int64_t N, const DropoutParams& d,
+                               hipStream_t s) {
+  size_t n4 = (size_t)M * N / 4;
+  if (n4 == 0) return hipSuccess;
+  size_t blocks = (n4 + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(dropout_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, mask, n4, d);
+  return hipGetLastError();
+}
+
+}  // namespace gmlp

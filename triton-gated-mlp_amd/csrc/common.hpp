@@ -1,0 +1,92 @@
+// Shared device helpers for the gfx950 gated-MLP kernels: storage types, MFMA wrappers,
+// fp32 SiLU, and the Philox4x32-10 counter RNG that defines the dropout mask.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gmlp {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Per-dtype traits.  An operand fragment of v_mfma_f32_32x32x16_{f16,bf16} is 8 consecutive
+// reduction elements per lane: lane l carries row (l % 32), reduction slots 8*(l / 32) .. +7.
+// The 16 accumulator floats of lane l sit at column (l % 32), rows 8*(i/4) + 4*(l/32) + (i%4).
+template <typename T>
+struct Traits;
+
+template <>
+struct Traits<f16> {
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_f32(f16 v) { return (float)v; }
+  static __device__ __forceinline__ f16 from_f32(float v) { return (f16)v; }
+};
+
+template <>
+struct Traits<bf16> {
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_f32(bf16 v) { return (float)v; }
+  static __device__ __forceinline__ bf16 from_f32(float v) { return (bf16)v; }
+};
+
+// sigma(x) = 1/(1+e^-x), silu(x) = x*sigma(x), silu'(x) = sigma*(1 + x*(1-sigma)); all fp32.
+// Same forms as the reference's _compute_sigma/_silu_fwd/_silu_bwd (src/triton_gated_mlp/ops/act.py:28-45).
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float silu_f32(float x) { return x * sigmoid_f32(x); }
+__device__ __forceinline__ float silu_grad_f32(float x) {
+  float s = sigmoid_f32(x);
+  return s * (1.0f + x * (1.0f - s));
+}
+
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
+__host__ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2,
+                                                        uint32_t c3, uint32_t k0, uint32_t k1,
+                                                        uint32_t out[4]) {
+  const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    uint64_t p0 = (uint64_t)M0 * c0;
+    uint64_t p1 = (uint64_t)M1 * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += W0; k1 += W1;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+struct DropoutParams {
+  uint32_t threshold;  // keep iff word >= threshold; threshold = floor(p * 2^32)
+  float scale;         // 1/(1-p)
+  uint32_t seed_lo, seed_hi, off_lo, off_hi;
+  int enabled;
+};
+
+// Keep bits for the 4 consecutive elements e4*4 .. e4*4+3 of the flattened [M,N] tensor.
+__host__ __device__ __forceinline__ void dropout_keep4(const DropoutParams& d, uint64_t e4,
+                                                        bool keep[4]) {
+  uint32_t w[4];
+  philox4x32_10((uint32_t)e4, (uint32_t)(e4 >> 32), d.off_lo, d.off_hi, d.seed_lo, d.seed_hi, w);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) keep[i] = w[i] >= d.threshold;
+}
+
+}  // namespace gmlp

@@ -1,0 +1,347 @@
+// LDS-tiled MFMA GEMM for gfx950 with pluggable operand orientation and fused epilogues.
+//
+//   C[M,N] (+)= sum over segments s, reduction k of  A_s[m,k] * B_s[n,k]
+//
+// Each operand is either reduction-contiguous ("KC": memory is [rows, K], K fastest) or
+// reduction-strided ("KS": memory is [K, rows], rows fastest).  The six GEMMs of the gated MLP
+// (gate/up, down, dH, dX, dW_gate/up, dW_down) are the combinations (KC,KC), (KC,KS), (KS,KS).
+// NB = 2 keeps two B operands and two accumulator sets per output element (gate and up share the
+// x tile), so the SiLU-gating epilogue sees both values in the same lane.
+//
+// Work decomposition: one workgroup (WGM x WGN wavefronts of 64 lanes) per BM x BN output tile,
+// each wavefront owning a (BM/WGM) x (BN/WGN) sub-tile as a grid of 32x32 MFMA accumulators.
+// Global memory -> registers -> LDS with two LDS stages; LDS rows of KC tiles are XOR-swizzled in
+// 16-byte chunks so that both the 16-byte stores and the ds_read_b128 fragment loads are free of
+// bank conflicts.  The MFMA is issued with operands swapped (B fragment as the instruction's A
+// operand), so a lane ends up with 4 consecutive output columns of one row: 8-byte stores.
+#pragma once
+#include "common.hpp"
+
+namespace gmlp {
+
+struct GemmArgs {
+  const void* A[2];  // per reduction segment
+  const void* B[2];  // per reduction segment (NB == 1) or per accumulator set (NB == 2)
+  int M, N, K;       // output rows, output cols, reduction length of one segment
+  int lda, ldb;      // leading dimensions (elements)
+  int nseg;          // number of reduction segments (1 or 2)
+  int group_m;       // tile-rows per scheduling group
+};
+
+// Workgroup id -> output tile.  The hardware deals consecutive workgroup ids round-robin to the
+// 8 XCDs (each with its own L2); undo that so each XCD walks a contiguous run of tiles, then walk
+// tiles in groups of `group_m` tile-rows (column-major inside a group) for operand reuse in L2.
+__device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tiles_n, int group_m,
+                                         int& tm, int& tn) {
+  const int NXCD = 8;
+  int xcd = pid % NXCD, loc = pid / NXCD;
+  int per = nwg / NXCD, rem = nwg % NXCD;
+  int t = xcd * per + (xcd < rem ? xcd : rem) + loc;
+  int in_group = group_m * tiles_n;
+  int gid = t / in_group;
+  int first_m = gid * group_m;
+  int gsz = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+  int r = t - gid * in_group;
+  tm = first_m + r % gsz;
+  tn = r / gsz;
+}
+
+template <int BK>
+__device__ __forceinline__ int swizzle_chunk(int row, int c) {
+  // 16 consecutive rows x one 16-byte chunk must hit 64 distinct banks.
+  if (BK == 64) return c ^ ((row >> 1) & 7);
+  return c ^ ((row >> 2) & 3);
+}
+
+// One operand tile: ROWS output-dimension rows by BK reduction elements.
+template <typename T, int ROWS, int BK, bool KS, int NT, bool EDGE>
+struct OperandTile {
+  typedef typename Traits<T>::vec8 vec8;
+  static constexpr int CHUNKS = ROWS * BK / 8;
+  static constexpr int PER_THREAD = CHUNKS / NT;
+  static_assert(CHUNKS % NT == 0, "tile chunks must divide evenly over the workgroup");
+  static constexpr int KS_LD = ROWS + 8;  // padded row length of a KS tile in LDS (elements)
+  static constexpr int LDS_ELEMS = KS ? BK * KS_LD : ROWS * BK;
+
+  uint4 regs[PER_THREAD];
+
+  // global -> registers.  r0: first output-dim row of the tile, k0: first reduction index.
+  __device__ __forceinline__ void gload(const T* __restrict__ p, int ld, int r0, int k0, int rtot,
+                                        int ktot, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      int q = tid + i * NT;
+      if (!KS) {
+        int row = q / (BK / 8), c = q % (BK / 8);
+        int gr = r0 + row, gk = k0 + c * 8;
+        bool ok = !EDGE || (gr < rtot && gk < ktot);
+        regs[i] = ok ? *(const uint4*)(p + (size_t)gr * ld + gk) : make_uint4(0, 0, 0, 0);
+      } else {
+        int krow = q / (ROWS / 8), c = q % (ROWS / 8);
+        int gk = k0 + krow, gr = r0 + c * 8;
+        bool ok = !EDGE || (gk < ktot && gr < rtot);
+        regs[i] = ok ? *(const uint4*)(p + (size_t)gk * ld + gr) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
+
+  // registers -> LDS
+  __device__ __forceinline__ void sstore(T* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      int q = tid + i * NT;
+      if (!KS) {
+        int row = q / (BK / 8), c = q % (BK / 8);
+        *(uint4*)(lds + row * BK + swizzle_chunk<BK>(row, c) * 8) = regs[i];
+      } else {
+        int krow = q / (ROWS / 8), c = q % (ROWS / 8);
+        *(uint4*)(lds + krow * KS_LD + c * 8) = regs[i];
+      }
+    }
+  }
+
+  // LDS -> MFMA fragment for the 32 rows starting at `row0`, reduction step `ks` (16 elements).
+  static __device__ __forceinline__ vec8 frag(const T* lds, int row0, int ks, int lane) {
+    int row = row0 + (lane & 31);
+    if (!KS) {
+      int c = ks * 2 + (lane >> 5);
+      return *(const vec8*)(lds + row * BK + swizzle_chunk<BK>(row, c) * 8);
+    } else {
+      vec8 f;
+      int kb = ks * 16 + 8 * (lane >> 5);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = lds[(kb + j) * KS_LD + row];
+      return f;
+    }
+  }
+};
+
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          bool EDGE>
+struct GemmConfig {
+  static constexpr int NT = WGM * WGN * 64;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  typedef OperandTile<T, BM, BK, A_KS, NT, EDGE> ATile;
+  typedef OperandTile<T, BN, BK, B_KS, NT, EDGE> BTile;
+  static constexpr int STAGE_ELEMS = ATile::LDS_ELEMS + NB * BTile::LDS_ELEMS;
+  static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * (int)sizeof(T);
+};
+
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          bool EDGE, typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64)
+    gemm_kernel(GemmArgs ga, typename Epi::Args ea) {
+  typedef GemmConfig<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE> Cfg;
+  typedef typename Cfg::ATile ATile;
+  typedef typename Cfg::BTile BTile;
+  typedef typename Traits<T>::vec8 vec8;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+
+  extern __shared__ __align__(16) char smem_raw[];
+  T* smem = (T*)smem_raw;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
+  int tm_i, tn_i;
+  map_tile(blockIdx.x, gridDim.x, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+
+  f32x16 acc[NB][TM][TN];
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
+
+  ATile at;
+  BTile bt[NB];
+
+  const int kt_seg = (ga.K + BK - 1) / BK;
+  const int kt_total = kt_seg * ga.nseg;
+
+  auto issue_loads = [&](int kt) {
+    int seg = kt / kt_seg;
+    int k0 = (kt - seg * kt_seg) * BK;
+    at.gload((const T*)ga.A[seg], ga.lda, m0, k0, ga.M, ga.K, tid);
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+      bt[b].gload((const T*)ga.B[NB == 2 ? b : seg], ga.ldb, n0, k0, ga.N, ga.K, tid);
+  };
+  auto commit = [&](int stage) {
+    T* s = smem + stage * Cfg::STAGE_ELEMS;
+    at.sstore(s, tid);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) bt[b].sstore(s + ATile::LDS_ELEMS + b * BTile::LDS_ELEMS, tid);
+  };
+
+  issue_loads(0);
+  commit(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < kt_total; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < kt_total) issue_loads(kt + 1);
+
+    const T* sa = smem + cur * Cfg::STAGE_ELEMS;
+    const T* sb = sa + ATile::LDS_ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      vec8 af[TM];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = ATile::frag(sa, wm * Cfg::WTM + i * 32, ks, lane);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          vec8 bf = BTile::frag(sb + b * BTile::LDS_ELEMS, wn * Cfg::WTN + j * 32, ks, lane);
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[b][i][j] = Traits<T>::mfma(bf, af[i], acc[b][i][j]);
+        }
+      }
+    }
+
+    if (kt + 1 < kt_total) commit(cur ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue: lane holds, for row m, 4 consecutive columns per group g.
+  const int mrow = lane & 31, nsub = 4 * (lane >> 5);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int m = m0 + wm * Cfg::WTM + i * 32 + mrow;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int n = n0 + wn * Cfg::WTN + j * 32 + 8 * g + nsub;
+        if (EDGE && (m >= ga.M || n >= ga.N)) continue;
+        f32x4 v0, v1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v0[r] = acc[0][i][j][4 * g + r];
+          v1[r] = acc[NB - 1][i][j][4 * g + r];
+        }
+        Epi::apply(ea, m, n, v0, v1);
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- epilogues
+
+template <typename T>
+__device__ __forceinline__ void store4(T* p, f32x4 v) {
+  typename Traits<T>::vec4 o;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) o[r] = Traits<T>::from_f32(v[r]);
+  *(typename Traits<T>::vec4*)p = o;
+}
+template <typename T>
+__device__ __forceinline__ f32x4 load4(const T* p) {
+  typename Traits<T>::vec4 o = *(const typename Traits<T>::vec4*)p;
+  f32x4 v;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) v[r] = Traits<T>::to_f32(o[r]);
+  return v;
+}
+
+// out = acc (+ bias[n])
+template <typename T>
+struct EpiStore {
+  struct Args {
+    T* out;
+    const T* bias;  // nullable
+    int ldc;
+  };
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 v, f32x4) {
+    if (a.bias) v += load4<T>(a.bias + n);
+    store4<T>(a.out + (size_t)m * a.ldc + n, v);
+  }
+};
+
+// G = acc0 + b_gate, U = acc1 + b_up, H = dropout(silu(G) * U)
+template <typename T>
+struct EpiGateUp {
+  struct Args {
+    T* h;
+    T* g_save;          // nullable
+    T* u_save;          // nullable
+    uint8_t* mask_out;  // nullable
+    const T* b_gate;    // nullable
+    const T* b_up;      // nullable
+    int ldc;
+    DropoutParams drop;
+  };
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 g, f32x4 u) {
+    if (a.b_gate) g += load4<T>(a.b_gate + n);
+    if (a.b_up) u += load4<T>(a.b_up + n);
+    size_t e = (size_t)m * a.ldc + n;
+    f32x4 h;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] = silu_f32(g[r]) * u[r];
+    if (a.drop.enabled) {
+      bool keep[4];
+      dropout_keep4(a.drop, e >> 2, keep);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
+      if (a.mask_out) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) packed |= (keep[r] ? 1u : 0u) << (8 * r);
+        *(uint32_t*)(a.mask_out + e) = packed;
+      }
+    } else if (a.mask_out) {
+      *(uint32_t*)(a.mask_out + e) = 0x01010101u;
+    }
+    store4<T>(a.h + e, h);
+    if (a.g_save) store4<T>(a.g_save + e, g);
+    if (a.u_save) store4<T>(a.u_save + e, u);
+  }
+};
+
+// Gating backward on 4 consecutive elements: dA = dH*keep/(1-p); dU = dA*silu(G); dG = dA*U*silu'(G)
+template <typename T>
+__device__ __forceinline__ void gating_bwd4(const DropoutParams& drop, size_t e, f32x4 dh,
+                                            const T* g, const T* u, T* dg, T* du) {
+  f32x4 gv = load4<T>(g + e), uv = load4<T>(u + e);
+  if (drop.enabled) {
+    bool keep[4];
+    dropout_keep4(drop, e >> 2, keep);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) dh[r] = keep[r] ? dh[r] * drop.scale : 0.f;
+  }
+  f32x4 dgv, duv;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float s = sigmoid_f32(gv[r]);
+    duv[r] = dh[r] * (gv[r] * s);
+    dgv[r] = dh[r] * uv[r] * (s * (1.0f + gv[r] * (1.0f - s)));
+  }
+  store4<T>(dg + e, dgv);
+  store4<T>(du + e, duv);
+}
+
+template <typename T>
+struct EpiDh {
+  struct Args {
+    const T* g;
+    const T* u;
+    T* dg;
+    T* du;
+    int ldc;
+    DropoutParams drop;
+  };
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 dh, f32x4) {
+    gating_bwd4<T>(a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
+  }
+};
+
+}  // namespace gmlp

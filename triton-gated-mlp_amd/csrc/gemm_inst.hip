@@ -1,0 +1,50 @@
+// One translation unit per (dtype, GEMM kind): compiled with -DGMLP_DT=<0|1> -DGMLP_KIND=<0..4>
+// so the kernels build in parallel.  Each unit instantiates the LARGE and MEDIUM tile classes.
+#include "launch.hpp"
+
+namespace gmlp {
+
+#if GMLP_DT == 0
+typedef f16 DT;
+#else
+typedef bf16 DT;
+#endif
+
+#define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
+  if (tile_class == TILE_LARGE)                                                                  \
+    return launch_gemm<DT, 256, BN_L, 64, 2, 2, AKS, BKS, NB, false, EPI<DT>>(ga, ea, s);         \
+  return launch_gemm<DT, 128, BN_M, 64, 2, 2, AKS, BKS, NB, true, EPI<DT>>(ga, ea, s);
+
+#if GMLP_KIND == 0
+template <>
+hipError_t launch_gateup<DT>(int tile_class, const GemmArgs& ga, const EpiGateUp<DT>::Args& ea,
+                             hipStream_t s) {
+  GMLP_DISPATCH(false, false, 2, EpiGateUp, 128, 64)
+}
+#elif GMLP_KIND == 1
+template <>
+hipError_t launch_linear<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>::Args& ea,
+                             hipStream_t s) {
+  GMLP_DISPATCH(false, false, 1, EpiStore, 256, 128)
+}
+#elif GMLP_KIND == 2
+template <>
+hipError_t launch_dh<DT>(int tile_class, const GemmArgs& ga, const EpiDh<DT>::Args& ea,
+                         hipStream_t s) {
+  GMLP_DISPATCH(false, true, 1, EpiDh, 256, 128)
+}
+#elif GMLP_KIND == 3
+template <>
+hipError_t launch_dx<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>::Args& ea,
+                         hipStream_t s) {
+  GMLP_DISPATCH(false, true, 1, EpiStore, 256, 128)
+}
+#elif GMLP_KIND == 4
+template <>
+hipError_t launch_dw<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>::Args& ea,
+                         hipStream_t s) {
+  GMLP_DISPATCH(true, true, 1, EpiStore, 256, 128)
+}
+#endif
+
+}  // namespace gmlp

@@ -1,0 +1,62 @@
+// Host-side launch interface between the C ABI (api.hip) and the kernel translation units.
+#pragma once
+#include "gemm.hpp"
+
+namespace gmlp {
+
+// Tile classes.  LARGE: 256x256x64 output tiles, 4 wavefronts of 128x128 (full tiles only).
+// MEDIUM: 128x128x64, 4 wavefronts of 64x64, with edge predication (any M, N%8, K%8).
+enum TileClass { TILE_LARGE = 0, TILE_MEDIUM = 1 };
+
+// kinds of GEMM the gated MLP needs; each is instantiated per dtype and tile class.
+template <typename T>
+hipError_t launch_gateup(int tile_class, const GemmArgs& ga, const typename EpiGateUp<T>::Args& ea,
+                         hipStream_t s);  // A KC, B KC, two accumulator sets
+template <typename T>
+hipError_t launch_linear(int tile_class, const GemmArgs& ga, const typename EpiStore<T>::Args& ea,
+                         hipStream_t s);  // A KC, B KC
+template <typename T>
+hipError_t launch_dh(int tile_class, const GemmArgs& ga, const typename EpiDh<T>::Args& ea,
+                     hipStream_t s);  // A KC, B KS
+template <typename T>
+hipError_t launch_dx(int tile_class, const GemmArgs& ga, const typename EpiStore<T>::Args& ea,
+                     hipStream_t s);  // A KC, B KS, two reduction segments
+template <typename T>
+hipError_t launch_dw(int tile_class, const GemmArgs& ga, const typename EpiStore<T>::Args& ea,
+                     hipStream_t s);  // A KS, B KS
+
+// Generic launcher used by the instantiation units.
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          bool EDGE, typename Epi>
+hipError_t launch_gemm(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
+  typedef GemmConfig<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE> Cfg;
+  auto kern = gemm_kernel<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE, Epi>;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
+  dim3 grid(tiles_m * tiles_n), block(Cfg::NT);
+  hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
+  return hipGetLastError();
+}
+
+// decode.hip
+template <typename T>
+hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
+                         const T* bu, const T* bd, T* h, T* y, int M, int K, int N, hipStream_t s);
+
+// aux.hip
+template <typename T>
+hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
+                             const DropoutParams& d, hipStream_t s);
+template <typename T>
+hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s);
+size_t colsum_workspace_bytes(int64_t M, int64_t C);
+hipError_t launch_dropout_mask(uint8_t* mask, int64_t M, int64_t N, const DropoutParams& d,
+                               hipStream_t s);
+
+}  // namespace gmlp

@@ -1,0 +1,123 @@
+"""ctypes binding of libgmlp.so (C ABI declared in include/gmlp.h).
+
+The library is the only implementation of the fused operators: if it cannot be found or loaded the
+import of the operators raises, there is no CPU or PyTorch fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+GMLP_F16, GMLP_BF16 = 0, 1
+GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM = 0, 1
+ABI_VERSION = 1
+
+_STATUS_EXC = {-1: ValueError, -2: NotImplementedError, -3: ValueError, -4: RuntimeError}
+
+_c_ptr = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_u64 = ctypes.c_uint64
+_int = ctypes.c_int
+_f32 = ctypes.c_float
+
+_SIGNATURES = {
+    "gmlp_abi_version": (_int, []),
+    "gmlp_last_error": (ctypes.c_char_p, []),
+    "gmlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
+    "gmlp_gateup_fwd": (_int, [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_dx_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_colsum": (_int, [_c_ptr] * 3 + [_i64, _i64, _int, _c_ptr]),
+    "gmlp_decode_fwd": (_int, [_c_ptr] * 10 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_dropout_mask": (_int, [_c_ptr, _i64, _i64, _f32, _u64, _u64, _c_ptr]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path() -> Path:
+    env = os.environ.get("GMLP_LIB")
+    if env:
+        return Path(env)
+    return Path(__file__).resolve().parent.parent / "lib" / "libgmlp.so"
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load libgmlp.so once; raise if it is missing (there is no other implementation)."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not path.exists():
+            raise RuntimeError(
+                f"libgmlp.so not found at {path}: build it with `make -C {path.parent.parent}` "
+                "(or set GMLP_LIB); the fused gated-MLP operators have no fallback path"
+            )
+        handle = ctypes.CDLL(str(path))
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = handle.gmlp_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"libgmlp.so ABI version {got}, expected {ABI_VERSION}")
+        _lib = handle
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = lib().gmlp_last_error().decode("utf-8", "replace")
+        raise _STATUS_EXC.get(status, RuntimeError)(msg)
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float16:
+        return GMLP_F16
+    if dtype == torch.bfloat16:
+        return GMLP_BF16
+    raise TypeError(
+        f"fused gated-MLP kernels take float16 or bfloat16 tensors, got {dtype}; "
+        "cast the module and its input (e.g. .to(torch.float16))"
+    )
+
+
+def require_gpu(*tensors: Optional[Tensor]) -> torch.device:
+    """All given tensors must live on one HIP device and share a dtype; returns the device."""
+    dev = None
+    dt = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "fused gated-MLP operators run on an AMD GPU only (tensor is on "
+                f"{t.device}); use EagerGatedMLP for CPU execution"
+            )
+        if dev is None:
+            dev, dt = t.device, t.dtype
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+        elif t.dtype != dt:
+            raise TypeError(f"tensors of different dtypes: {dt} and {t.dtype}")
+    assert dev is not None
+    return dev
+
+
+def ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

@@ -1,0 +1,211 @@
+"""Gated-MLP modules with the public surface of matteobonotto/triton-gated-mlp.
+
+  FusedGatedMLP(hidden_size, intermediate_size, bias, hidden_act, dropout_p)   nn.Module, HIP kernels
+  EagerGatedMLP(...)                                                           same math in plain torch
+  FusedGatedMLPFunction.apply(x, W_up, b_up, W_gp, b_gp)                       hidden-state autograd op
+  mlp_hidden_states_fwd / mlp_hidden_states_bwd, eager_fwd / eager_bwd, ACT_FWD
+
+Reference: src/triton_gated_mlp/gated_mlp.py (EagerGatedMLP :73-98, eager_fwd/bwd :105-156,
+FusedGatedMLPFunction :159-200, FusedGatedMLP :203-237).  Differences, all towards the eager
+semantics: the fused path applies the gate/up/down biases and dropout (the reference drops them),
+returns bias gradients, keeps G and U from the forward pass instead of recomputing them, and runs
+the down projection and its backward in the same kernels family (one autograd node for the MLP).
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor, nn
+from torch.autograd.function import Function
+
+from .ops import bwd as _bwd
+from .ops import fwd as _fwd
+from .ops.bwd import mlp_hidden_states_bwd
+from .ops.fwd import mlp_hidden_states_fwd
+
+ACT_FWD = {
+    "gelu": nn.GELU(),
+    "leaky_relu": nn.LeakyReLU(),
+    "relu": nn.ReLU(),
+    "sigmoid": nn.Sigmoid(),
+    "silu": nn.SiLU(),
+    "swish": nn.SiLU(),
+    "tanh": nn.Tanh(),
+    "no_act": nn.Identity(),
+}
+
+
+def _silu_op_bwd(x: Tensor, grad_output: Tensor) -> Tensor:
+    sigma = torch.sigmoid(x)
+    return grad_output * (sigma * (1 + x * (1 - sigma)))
+
+
+ACT_BWD = {"silu": _silu_op_bwd, "swish": _silu_op_bwd}
+
+
+class _GatedMLPBase(nn.Module):
+    """Parameters and attributes shared by the eager and the fused module (same names, same order)."""
+
+    def __init__(
+        self,
+        hidden_size: int = 256,
+        intermediate_size: int = 512,
+        bias: bool = True,
+        hidden_act: str = "silu",
+        dropout_p: float = 0.0,
+    ):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_proj = nn.Linear(hidden_size, intermediate_size, bias=bias)
+        self.up_proj = nn.Linear(hidden_size, intermediate_size, bias=bias)
+        self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=bias)
+        self.act = ACT_FWD[hidden_act]
+        self.act_fn = hidden_act
+        self.dropout = nn.Dropout(dropout_p)
+
+
+class EagerGatedMLP(_GatedMLPBase):
+    """down_proj(dropout(act(gate_proj(x)) * up_proj(x))) with stock torch operators."""
+
+    def forward(self, x: Tensor) -> Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        hidden = self.dropout(self.act(self.gate_proj(x2)) * self.up_proj(x2))
+        return self.down_proj(hidden).reshape(*lead, self.hidden_size)
+
+
+def eager_fwd(x: Tensor, WT_up: Tensor, b_up: Optional[Tensor], WT_gp: Tensor, b_gp: Optional[Tensor]) -> Tensor:
+    """silu(x·W_gpᵀ + b_gp) * (x·W_upᵀ + b_up) in plain torch."""
+    up = torch.nn.functional.linear(x, WT_up, b_up)
+    gate = torch.nn.functional.linear(x, WT_gp, b_gp)
+    return torch.nn.functional.silu(gate) * up
+
+
+def eager_bwd(x: Tensor, W_up: Tensor, W_gp: Tensor, grad_output: Tensor):
+    """Closed-form gradients (dx, dW_up, dW_gp) of eager_fwd without biases."""
+    up = x @ W_up.T
+    gate = x @ W_gp.T
+    d_up = grad_output * torch.nn.functional.silu(gate)
+    d_gate = _silu_op_bwd(gate, grad_output * up)
+    return d_up @ W_up + d_gate @ W_gp, d_up.T @ x, d_gate.T @ x
+
+
+class FusedGatedMLPFunction(Function):
+    """Hidden-state operator hidden = dropout(silu(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)).
+
+    Argument order (x, W_up, b_up, W_gp, b_gp) as in the reference; dropout_p/seed/offset are optional.
+    """
+
+    @staticmethod
+    def forward(ctx, x, W_up, b_up, W_gp, b_gp, dropout_p: float = 0.0, seed: int = 0, offset: int = 0):
+        needs_grad = any(ctx.needs_input_grad[:5])
+        out = _fwd.gateup_fwd(x, W_gp, b_gp, W_up, b_up, dropout_p, seed, offset, save_activations=needs_grad)
+        if needs_grad:
+            ctx.save_for_backward(x, W_up, W_gp, out.gate, out.up)
+        ctx.dropout = (float(dropout_p), int(seed), int(offset))
+        ctx.has_bias = (b_up is not None, b_gp is not None)
+        return out.hidden
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, W_up, W_gp, gate, up = ctx.saved_tensors
+        p, seed, offset = ctx.dropout
+        need = ctx.needs_input_grad
+        dg, du = _bwd.gating_bwd(grad_output, gate, up, p, seed, offset)
+        dx = _bwd.dx_bwd(dg, du, W_gp, W_up) if need[0] else None
+        dW_up = _bwd.dw_bwd(du, x) if need[1] else None
+        db_up = _bwd.colsum(du) if ctx.has_bias[0] and need[2] else None
+        dW_gp = _bwd.dw_bwd(dg, x) if need[3] else None
+        db_gp = _bwd.colsum(dg) if ctx.has_bias[1] and need[4] else None
+        grads = (dx, dW_up, db_up, dW_gp, db_gp, None, None, None)
+        return grads[: len(need)]  # apply() may have been called with the 5 reference arguments only
+
+
+class FusedGatedMLPFullFunction(Function):
+    """Whole MLP as one autograd node, so dY -> (dG, dU) is a single GEMM with a fused epilogue."""
+
+    @staticmethod
+    def forward(ctx, x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset):
+        needs_grad = any(ctx.needs_input_grad[:7])
+        hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=needs_grad)
+        y = _fwd.linear_fwd(hs.hidden, W_down, b_down)
+        if needs_grad:
+            ctx.save_for_backward(x, W_gate, W_up, W_down, hs.gate, hs.up, hs.hidden)
+        ctx.dropout = (float(dropout_p), int(seed), int(offset))
+        ctx.has_bias = (b_gate is not None, b_up is not None, b_down is not None)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, W_gate, W_up, W_down, gate, up, hidden = ctx.saved_tensors
+        p, seed, offset = ctx.dropout
+        need = ctx.needs_input_grad
+        dy = dy.contiguous()
+        dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
+        if any(need[:5]):
+            dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset)
+            if need[0]:
+                dx = _bwd.dx_bwd(dg, du, W_gate, W_up)
+            if need[1]:
+                dW_gate = _bwd.dw_bwd(dg, x)
+            if ctx.has_bias[0] and need[2]:
+                db_gate = _bwd.colsum(dg)
+            if need[3]:
+                dW_up = _bwd.dw_bwd(du, x)
+            if ctx.has_bias[1] and need[4]:
+                db_up = _bwd.colsum(du)
+        if need[5]:
+            dW_down = _bwd.dw_bwd(dy, hidden)
+        if ctx.has_bias[2] and need[6]:
+            db_down = _bwd.colsum(dy)
+        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None
+
+
+class FusedGatedMLP(_GatedMLPBase):
+    """Drop-in gated MLP running on hand-written gfx950 kernels (float16 / bfloat16).
+
+    Dropout is active in training mode only.  The keep mask comes from a counter-based generator:
+    set `dropout_seed` (int) for a fixed mask stream, otherwise each forward draws a seed from
+    torch's default CPU generator (so `torch.manual_seed` makes runs repeatable).  The seed and
+    offset of the last training forward are kept in `last_dropout_state`.
+    """
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        if self.act_fn not in ("silu", "swish"):
+            raise NotImplementedError(
+                f"FusedGatedMLP implements hidden_act='silu' only, got {self.act_fn!r}; use EagerGatedMLP"
+            )
+        self.dropout_seed: Optional[int] = None
+        self._dropout_calls = 0
+        self.last_dropout_state = (0, 0)
+
+    def _next_dropout_state(self):
+        if self.dropout_seed is None:
+            seed, offset = int(torch.randint(0, 2**62, (1,)).item()), 0
+        else:
+            seed, offset = int(self.dropout_seed), self._dropout_calls
+            self._dropout_calls += 1
+        self.last_dropout_state = (seed, offset)
+        return seed, offset
+
+    def forward(self, x: Tensor) -> Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        p = float(self.dropout.p) if self.training else 0.0
+        gate, up, down = self.gate_proj, self.up_proj, self.down_proj
+        M, K = x2.shape
+        inference = not torch.is_grad_enabled() or not (
+            x2.requires_grad or any(q.requires_grad for q in self.parameters())
+        )
+        if inference and p == 0.0 and _fwd.decode_supported(M, K, self.intermediate_size):
+            y = _fwd.decode_fwd(x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias)
+        else:
+            seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
+            y = FusedGatedMLPFullFunction.apply(
+                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p, seed, offset
+            )
+        return y.reshape(*lead, self.hidden_size)

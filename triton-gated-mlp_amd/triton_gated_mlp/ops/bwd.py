@@ -1,0 +1,157 @@
+"""Backward operators of the gated MLP on MI355X (host wrappers over libgmlp.so).
+
+`mlp_hidden_states_bwd(x, W_up, W_gp, grad_output)` keeps the reference signature and return
+order `(dx, dW_up, dW_gp)` (src/triton_gated_mlp/ops/bwd.py:466-468,602).  The reference
+recomputes G and U inside its first backward kernel; callers that kept them from the forward pass
+hand them in through the keyword arguments and skip that GEMM.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from .. import _cabi
+from .fwd import _c, gateup_fwd
+
+
+def dh_bwd(
+    dy: Tensor, W_down: Tensor, g: Tensor, u: Tensor, dropout_p: float = 0.0, seed: int = 0, offset: int = 0
+) -> Tuple[Tensor, Tensor]:
+    """(dG, dU) from dY: dH = dY·W_down with dropout and gating backward fused in the epilogue."""
+    M, K = dy.shape
+    N = W_down.shape[1]
+    if tuple(W_down.shape) != (K, N) or tuple(g.shape) != (M, N) or tuple(u.shape) != (M, N):
+        raise ValueError("dimension mismatch among dy, W_down, g, u")
+    dev = _cabi.require_gpu(dy, W_down, g, u)
+    code = _cabi.dtype_code(dy.dtype)
+    dy, W_down, g, u = _c(dy), _c(W_down), _c(g), _c(u)
+    dg = torch.empty_like(g)
+    du = torch.empty_like(u)
+    if M > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_dh_bwd(
+                    _cabi.ptr(dy), _cabi.ptr(W_down), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du),
+                    M, K, N, code, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                )
+            )
+    return dg, du
+
+
+def gating_bwd(
+    dh: Tensor, g: Tensor, u: Tensor, dropout_p: float = 0.0, seed: int = 0, offset: int = 0
+) -> Tuple[Tensor, Tensor]:
+    """(dG, dU) from dH (element-wise): dU = dA*silu(G), dG = dA*U*silu'(G), dA = dH*keep/(1-p)."""
+    if g.shape != dh.shape or u.shape != dh.shape or dh.ndim != 2:
+        raise ValueError("dh, g, u must be 2-D tensors of one shape")
+    dev = _cabi.require_gpu(dh, g, u)
+    code = _cabi.dtype_code(dh.dtype)
+    dh, g, u = _c(dh), _c(g), _c(u)
+    M, N = dh.shape
+    dg = torch.empty_like(g)
+    du = torch.empty_like(u)
+    if M > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_gating_bwd(
+                    _cabi.ptr(dh), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du), M, N, code,
+                    float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                )
+            )
+    return dg, du
+
+
+def dx_bwd(dg: Tensor, du: Tensor, W_gate: Tensor, W_up: Tensor) -> Tensor:
+    """dX = dG·W_gate + dU·W_up as one GEMM over the concatenated reduction."""
+    M, N = dg.shape
+    K = W_gate.shape[1]
+    if du.shape != dg.shape or tuple(W_gate.shape) != (N, K) or tuple(W_up.shape) != (N, K):
+        raise ValueError("dimension mismatch among dg, du, W_gate, W_up")
+    dev = _cabi.require_gpu(dg, du, W_gate, W_up)
+    code = _cabi.dtype_code(dg.dtype)
+    dg, du, W_gate, W_up = _c(dg), _c(du), _c(W_gate), _c(W_up)
+    dx = torch.empty((M, K), dtype=dg.dtype, device=dev)
+    if M > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_dx_bwd(
+                    _cabi.ptr(dg), _cabi.ptr(du), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(dx), M, K, N,
+                    code, _cabi.stream_ptr(dev),
+                )
+            )
+    return dx
+
+
+def dw_bwd(lhs: Tensor, rhs: Tensor) -> Tensor:
+    """dW[R,C] = lhs[M,R]ᵀ · rhs[M,C] (weight gradient of a linear layer)."""
+    if lhs.ndim != 2 or rhs.ndim != 2 or lhs.shape[0] != rhs.shape[0]:
+        raise ValueError(f"dimension mismatch: lhs {tuple(lhs.shape)}, rhs {tuple(rhs.shape)}")
+    dev = _cabi.require_gpu(lhs, rhs)
+    code = _cabi.dtype_code(lhs.dtype)
+    lhs, rhs = _c(lhs), _c(rhs)
+    M, R = lhs.shape
+    C = rhs.shape[1]
+    if M == 0:
+        return torch.zeros((R, C), dtype=lhs.dtype, device=dev)
+    dw = torch.empty((R, C), dtype=lhs.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_dw_bwd(
+                _cabi.ptr(lhs), _cabi.ptr(rhs), _cabi.ptr(dw), M, R, C, code, _cabi.stream_ptr(dev)
+            )
+        )
+    return dw
+
+
+def colsum(a: Tensor) -> Tensor:
+    """Σ_m a[m,:] with fp32 accumulation in a fixed order (bias gradient)."""
+    if a.ndim != 2:
+        raise ValueError("colsum takes a 2-D tensor")
+    dev = _cabi.require_gpu(a)
+    code = _cabi.dtype_code(a.dtype)
+    a = _c(a)
+    M, C = a.shape
+    if M == 0:
+        return torch.zeros((C,), dtype=a.dtype, device=dev)
+    out = torch.empty((C,), dtype=a.dtype, device=dev)
+    nbytes = _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, M, 0, C, code)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_colsum(_cabi.ptr(a), _cabi.ptr(out), _cabi.ptr(ws), M, C, code, _cabi.stream_ptr(dev))
+        )
+    return out
+
+
+def mlp_hidden_states_bwd(
+    x: Tensor,
+    W_up: Tensor,
+    W_gp: Tensor,
+    grad_output: Tensor,
+    *,
+    b_up: Optional[Tensor] = None,
+    b_gp: Optional[Tensor] = None,
+    gate: Optional[Tensor] = None,
+    up: Optional[Tensor] = None,
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    return_bias_grads: bool = False,
+):
+    """Gradients of hidden = dropout(silu(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)) w.r.t. x, W_up, W_gp.
+
+    Returns (dx, dW_up, dW_gp), or (dx, dW_up, db_up, dW_gp, db_gp) with return_bias_grads.
+    """
+    if gate is None or up is None:
+        fwd = gateup_fwd(x, W_gp, b_gp, W_up, b_up, 0.0, 0, 0, save_activations=True)
+        gate, up = fwd.gate, fwd.up
+    dg, du = gating_bwd(grad_output, gate, up, dropout_p, seed, offset)
+    dx = dx_bwd(dg, du, W_gp, W_up)
+    dW_up = dw_bwd(du, x)
+    dW_gp = dw_bwd(dg, x)
+    if return_bias_grads:
+        return dx, dW_up, colsum(du), dW_gp, colsum(dg)
+    return dx, dW_up, dW_gp

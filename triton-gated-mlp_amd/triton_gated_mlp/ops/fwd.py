@@ -1,0 +1,172 @@
+"""Forward operators of the gated MLP on MI355X (host wrappers over libgmlp.so).
+
+`mlp_hidden_states_fwd` keeps the positional signature of the reference operator
+(src/triton_gated_mlp/ops/fwd.py:198-206); the keyword-only arguments are extensions (dropout seed,
+saving G and U for the backward pass).  Unlike the reference it applies the biases and the dropout
+it is given, and makes its inputs contiguous instead of assuming it.
+"""
+
+from __future__ import annotations
+
+from typing import NamedTuple, Optional
+
+import torch
+from torch import Tensor
+
+from .. import _cabi
+
+
+def validate_dimensions(
+    x: Tensor, WT_up: Tensor, b_up: Optional[Tensor], WT_gp: Tensor, b_gp: Optional[Tensor]
+) -> None:
+    """Same conditions as the reference (src/triton_gated_mlp/ops/fwd.py:169-184), raised as ValueError."""
+    if x.ndim != 2:
+        raise ValueError(f"input tensor must be 2-D [M, K], got {x.ndim} dims")
+    if WT_up.ndim != 2 or WT_up.shape[1] != x.shape[1]:
+        raise ValueError(f"dimension mismatch in WT_up {tuple(WT_up.shape)} or x {tuple(x.shape)}")
+    if WT_gp.shape != WT_up.shape:
+        raise ValueError(f"dimension mismatch in WT_up {tuple(WT_up.shape)} or WT_gp {tuple(WT_gp.shape)}")
+    if b_up is not None and tuple(b_up.shape) != (WT_up.shape[0],):
+        raise ValueError("dimension mismatch in b_up")
+    if b_gp is not None and tuple(b_gp.shape) != (WT_up.shape[0],):
+        raise ValueError("dimension mismatch in b_gp")
+
+
+class HiddenStates(NamedTuple):
+    hidden: Tensor
+    gate: Optional[Tensor]  # G = x·W_gateᵀ + b_gate (kept for backward)
+    up: Optional[Tensor]  # U = x·W_upᵀ + b_up
+    mask: Optional[Tensor]  # uint8 keep mask
+
+
+def _c(t: Optional[Tensor]) -> Optional[Tensor]:
+    return None if t is None else t.contiguous()
+
+
+def gateup_fwd(
+    x: Tensor,
+    W_gate: Tensor,
+    b_gate: Optional[Tensor],
+    W_up: Tensor,
+    b_up: Optional[Tensor],
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    save_activations: bool = False,
+    return_mask: bool = False,
+) -> HiddenStates:
+    """H = dropout(silu(x·W_gateᵀ + b_gate) * (x·W_upᵀ + b_up)) in one kernel."""
+    validate_dimensions(x, W_up, b_up, W_gate, b_gate)
+    dev = _cabi.require_gpu(x, W_gate, b_gate, W_up, b_up)
+    code = _cabi.dtype_code(x.dtype)
+    x, W_gate, W_up, b_gate, b_up = _c(x), _c(W_gate), _c(W_up), _c(b_gate), _c(b_up)
+    M, K = x.shape
+    N = W_up.shape[0]
+    h = torch.empty((M, N), dtype=x.dtype, device=dev)
+    g = torch.empty_like(h) if save_activations else None
+    u = torch.empty_like(h) if save_activations else None
+    mask = torch.empty((M, N), dtype=torch.uint8, device=dev) if return_mask else None
+    if M > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_gateup_fwd(
+                    _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(b_gate), _cabi.ptr(b_up),
+                    _cabi.ptr(h), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(mask),
+                    M, K, N, code, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                )
+            )
+    return HiddenStates(h, g, u, mask)
+
+
+def mlp_hidden_states_fwd(
+    x: Tensor,
+    WT_up: Tensor,
+    b_up: Optional[Tensor],
+    WT_gp: Tensor,
+    b_gp: Optional[Tensor],
+    act_fn: str = "silu",
+    dropout_p: float = 0.0,
+    *,
+    seed: int = 0,
+    offset: int = 0,
+) -> Tensor:
+    """dropout(act_fn(gate_proj(x)) * up_proj(x)) fused; weights in nn.Linear [N, K] layout."""
+    if act_fn not in ("silu", "swish"):
+        raise NotImplementedError(f"fused gated MLP supports act_fn='silu' only, got {act_fn!r}")
+    return gateup_fwd(x, WT_gp, b_gp, WT_up, b_up, dropout_p, seed, offset).hidden
+
+
+def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
+    """a[M,R]·W[C,R]ᵀ + bias: the down projection (reference: nn.Linear, gated_mlp.py:236)."""
+    if a.ndim != 2 or W.ndim != 2 or W.shape[1] != a.shape[1]:
+        raise ValueError(f"dimension mismatch: a {tuple(a.shape)}, W {tuple(W.shape)}")
+    if bias is not None and tuple(bias.shape) != (W.shape[0],):
+        raise ValueError("dimension mismatch in bias")
+    dev = _cabi.require_gpu(a, W, bias)
+    code = _cabi.dtype_code(a.dtype)
+    a, W, bias = _c(a), _c(W), _c(bias)
+    M, R = a.shape
+    C = W.shape[0]
+    out = torch.empty((M, C), dtype=a.dtype, device=dev)
+    if M > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_linear_fwd(
+                    _cabi.ptr(a), _cabi.ptr(W), _cabi.ptr(bias), _cabi.ptr(out), M, R, C, code,
+                    _cabi.stream_ptr(dev),
+                )
+            )
+    return out
+
+
+DECODE_MAX_M = 16
+
+
+def decode_supported(M: int, K: int, N: int) -> bool:
+    return 1 <= M <= DECODE_MAX_M and K % 32 == 0 and N % 256 == 0
+
+
+def decode_fwd(
+    x: Tensor,
+    W_gate: Tensor,
+    b_gate: Optional[Tensor],
+    W_up: Tensor,
+    b_up: Optional[Tensor],
+    W_down: Tensor,
+    b_down: Optional[Tensor],
+) -> Tensor:
+    """Whole-MLP forward for M <= 16 token rows: every weight byte is read from HBM once."""
+    validate_dimensions(x, W_up, b_up, W_gate, b_gate)
+    M, K = x.shape
+    N = W_up.shape[0]
+    if tuple(W_down.shape) != (K, N):
+        raise ValueError(f"dimension mismatch in W_down {tuple(W_down.shape)}")
+    dev = _cabi.require_gpu(x, W_gate, b_gate, W_up, b_up, W_down, b_down)
+    code = _cabi.dtype_code(x.dtype)
+    x, W_gate, W_up, W_down = _c(x), _c(W_gate), _c(W_up), _c(W_down)
+    b_gate, b_up, b_down = _c(b_gate), _c(b_up), _c(b_down)
+    h = torch.empty((M, N), dtype=x.dtype, device=dev)
+    y = torch.empty((M, K), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_decode_fwd(
+                _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(W_down), _cabi.ptr(b_gate),
+                _cabi.ptr(b_up), _cabi.ptr(b_down), _cabi.ptr(h), _cabi.ptr(y), None, M, K, N, code,
+                _cabi.stream_ptr(dev),
+            )
+        )
+    return y
+
+
+def dropout_mask(M: int, N: int, dropout_p: float, seed: int, offset: int = 0, device=None) -> Tensor:
+    """uint8 [M,N] keep mask of the kernels' counter-based generator (1 = keep)."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    mask = torch.empty((M, N), dtype=torch.uint8, device=dev)
+    if M * N > 0:
+        with torch.cuda.device(dev):
+            _cabi.check(
+                _cabi.lib().gmlp_dropout_mask(
+                    _cabi.ptr(mask), M, N, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev)
+                )
+            )
+    return mask
