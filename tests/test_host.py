@@ -1,0 +1,166 @@
+"""Host-side checks that need no GPU: the C ABI loads and exports what include/gmlp.h declares,
+argument validation returns error codes before any device work, and the Python surface mirrors the
+reference's module/operator interface."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+
+from triton_gated_mlp import _cabi  # noqa: E402
+import triton_gated_mlp as tgm  # noqa: E402
+from triton_gated_mlp.gated_mlp import ACT_FWD, EagerGatedMLP, FusedGatedMLP  # noqa: E402
+from triton_gated_mlp.utils import copy_weights, get_device  # noqa: E402
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "gmlp.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gmlp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _cabi.lib()
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f"libgmlp.so does not export {name}"
+    assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
+    assert lib.gmlp_abi_version() == 1
+
+
+def _buf(nbytes=4096):
+    raw = ctypes.create_string_buffer(nbytes + 64)
+    addr = (ctypes.addressof(raw) + 63) & ~63
+    return raw, addr
+
+
+def test_argument_validation_returns_codes_without_touching_the_device():
+    lib = _cabi.lib()
+    _, a = _buf()
+    err = lambda: lib.gmlp_last_error().decode()
+    # NULL pointer
+    assert lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None) == -1 and "NULL" in err()
+    # bad dtype
+    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 8, 8, 7, None) == -1 and "dtype" in err()
+    # shape: K not a multiple of 8, M < 1
+    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None) == -2 and "multiple of 8" in err()
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0.0, 0, 0, None) == -2
+    # alignment
+    assert lib.gmlp_linear_fwd(a + 2, a, None, a, 8, 8, 8, 0, None) == -3 and "aligned" in err()
+    # dropout probability outside [0, 1)
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 1.0, 0, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, -0.1, 0, 0, None) == -1
+    assert lib.gmlp_dropout_mask(a, 8, 8, float("nan"), 0, 0, None) == -1
+    # decode limits
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 17, 256, 256, 0, None) == -2 and "16" in err()
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 40, 256, 0, None) == -2
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 128, 0, None) == -2
+    for fn, args in [
+        (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0.0, 0, 0, None)),
+        (lib.gmlp_gating_bwd, (a, a, a, a, None, 8, 8, 0, 0.0, 0, 0, None)),
+        (lib.gmlp_dx_bwd, (a, a, a, a, None, 8, 8, 8, 0, None)),
+        (lib.gmlp_dw_bwd, (a, None, a, 8, 8, 8, 0, None)),
+        (lib.gmlp_colsum, (a, a, None, 8, 8, 0, None)),
+    ]:
+        assert fn(*args) == -1
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, 100, 0, 64, 0) == 64 * 64 * 4
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DECODE_FWD, 16, 8192, 28672, 0) == 0
+
+
+def test_error_codes_map_to_python_exceptions():
+    lib = _cabi.lib()
+    _, a = _buf()
+    with pytest.raises(NotImplementedError, match="multiple of 8"):
+        _cabi.check(lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None))
+    with pytest.raises(ValueError, match="NULL"):
+        _cabi.check(lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None))
+    with pytest.raises(TypeError, match="float16 or bfloat16"):
+        _cabi.dtype_code(torch.float32)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setenv("GMLP_LIB", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_cabi, "_lib", None)
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _cabi.lib()
+
+
+def test_module_surface_matches_reference():
+    """ctor kwargs, attributes and parameter names of src/triton_gated_mlp/gated_mlp.py:203-220."""
+    m = FusedGatedMLP(hidden_size=64, intermediate_size=128, dropout_p=0.1, bias=True)
+    names = [n for n, _ in m.named_parameters()]
+    assert names == ["gate_proj.weight", "gate_proj.bias", "up_proj.weight", "up_proj.bias", "down_proj.weight",
+                     "down_proj.bias"]
+    assert m.gate_proj.weight.shape == (128, 64) and m.down_proj.weight.shape == (64, 128)
+    assert m.hidden_size == 64 and m.intermediate_size == 128 and m.act_fn == "silu" and m.dropout.p == 0.1
+    assert isinstance(m.act, torch.nn.SiLU)
+    d = FusedGatedMLP()
+    assert (d.hidden_size, d.intermediate_size, d.dropout.p) == (256, 512, 0.0) and d.gate_proj.bias is not None
+    assert [n for n, _ in FusedGatedMLP(bias=False).named_parameters()] == [
+        "gate_proj.weight", "up_proj.weight", "down_proj.weight"]
+    assert set(ACT_FWD) >= {"silu", "swish", "gelu", "relu", "no_act"}
+    with pytest.raises(NotImplementedError):
+        FusedGatedMLP(hidden_act="gelu")
+    for name in ("EagerGatedMLP", "FusedGatedMLP", "FusedGatedMLPFunction", "mlp_hidden_states_fwd",
+                 "mlp_hidden_states_bwd", "eager_fwd", "eager_bwd", "ACT_FWD"):
+        assert hasattr(tgm.gated_mlp, name)
+
+
+def test_state_dict_interchange_and_copy_weights():
+    torch.manual_seed(0)
+    e = EagerGatedMLP(32, 64, bias=True)
+    f = FusedGatedMLP(32, 64, bias=True)
+    f.load_state_dict(e.state_dict())
+    for (n1, p1), (n2, p2) in zip(e.named_parameters(), f.named_parameters()):
+        assert n1 == n2 and torch.equal(p1, p2)
+    g = FusedGatedMLP(32, 64, bias=True)
+    copy_weights(e, g)
+    assert all(torch.equal(a, b) for a, b in zip(e.parameters(), g.parameters()))
+    assert g.gate_proj.weight.data_ptr() != e.gate_proj.weight.data_ptr()
+    assert get_device().type in ("cpu", "cuda")
+
+
+def test_fused_module_has_no_cpu_path():
+    m = FusedGatedMLP(64, 128).half()
+    with pytest.raises(RuntimeError, match="AMD GPU only"):
+        m(torch.randn(4, 64).half())
+
+
+def test_eager_module_semantics_on_cpu():
+    from oracle import eager as oracle
+
+    torch.manual_seed(1)
+    e = EagerGatedMLP(16, 24, bias=True).double()
+    x = torch.randn(2, 5, 16, dtype=torch.float64)
+    y = e(x)
+    ref = oracle.forward(x.view(-1, 16), e.gate_proj.weight, e.gate_proj.bias, e.up_proj.weight, e.up_proj.bias,
+                         e.down_proj.weight, e.down_proj.bias)["Y"]
+    assert y.shape == x.shape and torch.allclose(y.view(-1, 16), ref, atol=1e-12)
+    t = torch.randn(7, 16, dtype=torch.float64)
+    Wu, Wg, dH = e.up_proj.weight.detach(), e.gate_proj.weight.detach(), torch.randn(7, 24, dtype=torch.float64)
+    h = tgm.eager_fwd(t, Wu, None, Wg, None)
+    assert torch.allclose(h, oracle.hidden_forward(t, Wg, None, Wu, None)["H"], atol=1e-12)
+    dx, dWu, dWg = tgm.eager_bwd(t, Wu, Wg, dH)
+    hb = oracle.hidden_backward(dH, t @ Wg.T, t @ Wu.T)
+    assert torch.allclose(dx, hb["dU"] @ Wu + hb["dG"] @ Wg, atol=1e-12)
+    assert torch.allclose(dWu, hb["dU"].T @ t, atol=1e-12) and torch.allclose(dWg, hb["dG"].T @ t, atol=1e-12)
+
+
+def test_operator_shape_validation_happens_before_device_checks():
+    from triton_gated_mlp.ops.fwd import validate_dimensions
+
+    x, W = torch.zeros(4, 16), torch.zeros(8, 16)
+    validate_dimensions(x, W, None, W, None)
+    with pytest.raises(ValueError):
+        validate_dimensions(torch.zeros(2, 4, 16), W, None, W, None)
+    with pytest.raises(ValueError):
+        validate_dimensions(x, torch.zeros(8, 12), None, W, None)
+    with pytest.raises(ValueError):
+        validate_dimensions(x, W, torch.zeros(7), W, None)
+    with pytest.raises(NotImplementedError):
+        tgm.mlp_hidden_states_fwd(x, W, None, W, None, "gelu", 0.0)
