@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 
 #include "launch.hpp"
 
@@ -72,8 +73,10 @@ int hip_result(const char* fn, hipError_t e) {
 // tiles to occupy the chip; everything else runs on the predicated MEDIUM class.
 int pick_tile(int64_t rows, int64_t cols, int64_t red, int bn_large) {
   if (rows % 256 == 0 && cols % bn_large == 0 && red % 64 == 0 &&
-      (rows / 256) * (cols / bn_large) >= 192)
-    return gmlp::TILE_LARGE;
+      (rows / 256) * (cols / bn_large) >= 192) {
+    static const bool v1 = getenv("GMLP_FORCE_V1") != nullptr;
+    return v1 ? gmlp::TILE_LARGE_V1 : gmlp::TILE_LARGE;
+  }
   return gmlp::TILE_MEDIUM;
 }
 

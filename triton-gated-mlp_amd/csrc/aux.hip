@@ -7,23 +7,25 @@ namespace gmlp {
 template <typename T>
 __global__ void __launch_bounds__(256)
     gating_bwd_kernel(const T* __restrict__ dh, const T* __restrict__ g, const T* __restrict__ u,
-                      T* __restrict__ dg, T* __restrict__ du, size_t n4, DropoutParams d) {
+                      T* __restrict__ dg, T* __restrict__ du, size_t n8, DropoutParams d) {
   size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    size_t e = i * 4;
-    gating_bwd4<T>(d, e, load4<T>(dh + e), g, u, dg, du);
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+    size_t e = i * 8;
+    float v[8];
+    load_w<T, 8>(dh + e, v);
+    gating_bwd_w<T, 8>(d, e, v, g, u, dg, du);
   }
 }
 
 template <typename T>
 hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
                              const DropoutParams& d, hipStream_t s) {
-  size_t n4 = (size_t)M * N / 4;
-  if (n4 == 0) return hipSuccess;
-  size_t blocks = (n4 + 255) / 256;
+  size_t n8 = (size_t)M * N / 8;
+  if (n8 == 0) return hipSuccess;
+  size_t blocks = (n8 + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
   hipLaunchKernelGGL(gating_bwd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, dh, g, u, dg, du,
-                     n4, d);
+                     n8, d);
   return hipGetLastError();
 }
 template hipError_t launch_gating_bwd<f16>(const f16*, const f16*, const f16*, f16*, f16*, int64_t,
@@ -42,7 +44,12 @@ __global__ void __launch_bounds__(256)
   int64_t rows = (M + COLSUM_SPLITS - 1) / COLSUM_SPLITS;
   int64_t r0 = blockIdx.y * rows, r1 = r0 + rows < M ? r0 + rows : M;
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t r = r0; r < r1; ++r) s += load4<T>(a + r * C + c);
+  for (int64_t r = r0; r < r1; ++r) {
+    float t[4];
+    load_w<T, 4>(a + r * C + c, t);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) s[q] += t[q];
+  }
   *(f32x4*)(ws + (int64_t)blockIdx.y * C + c) = s;
 }
 
@@ -53,7 +60,8 @@ __global__ void __launch_bounds__(256)
   if (c >= C) return;
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
   for (int i = 0; i < COLSUM_SPLITS; ++i) s += *(const f32x4*)(ws + (int64_t)i * C + c);
-  store4<T>(out + c, s);
+  float t[4] = {s[0], s[1], s[2], s[3]};
+  store_w<T, 4>(out + c, t);
 }
 
 size_t colsum_workspace_bytes(int64_t, int64_t C) { return (size_t)COLSUM_SPLITS * C * sizeof(float); }

@@ -112,14 +112,14 @@ __global__ void __launch_bounds__(256)
   // lane holds token row m = lane%16, hidden columns n = nb*16 + 4*(lane/16) + r
   if (mok) {
     int n = nb * 16 + 4 * kg;
-    f32x4 g, u, hv;
+    float g[4], u[4], hv[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) { g[r] = accg[r]; u[r] = accu[r]; }
-    if (bg) g += load4<T>(bg + n);
-    if (bu) u += load4<T>(bu + n);
+    if (bg) add_w<T, 4>(bg + n, g);
+    if (bu) add_w<T, 4>(bu + n, u);
 #pragma unroll
     for (int r = 0; r < 4; ++r) hv[r] = silu_f32(g[r]) * u[r];
-    store4<T>(h + (size_t)r16 * N + n, hv);
+    store_w<T, 4>(h + (size_t)r16 * N + n, hv);
   }
 }
 
@@ -186,14 +186,14 @@ __global__ void __launch_bounds__(DEC_SPLIT * 64)
   for (int r = 0; r < 4; ++r) part[w][lane][r] = acc[r];
   __syncthreads();
   if (w == 0 && mok) {
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < DEC_SPLIT; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) s[r] += part[i][lane][r];
     int c = cb * 16 + 4 * kg;
-    if (bd) s += load4<T>(bd + c);
-    store4<T>(y + (size_t)r16 * K + c, s);
+    if (bd) add_w<T, 4>(bd + c, s);
+    store_w<T, 4>(y + (size_t)r16 * K + c, s);
   }
 }
 

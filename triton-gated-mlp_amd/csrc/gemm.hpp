@@ -223,34 +223,53 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
       for (int g = 0; g < 4; ++g) {
         int n = n0 + wn * Cfg::WTN + j * 32 + 8 * g + nsub;
         if (EDGE && (m >= ga.M || n >= ga.N)) continue;
-        f32x4 v0, v1;
+        float v0[4], v1[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           v0[r] = acc[0][i][j][4 * g + r];
           v1[r] = acc[NB - 1][i][j][4 * g + r];
         }
-        Epi::apply(ea, m, n, v0, v1);
+        Epi::template apply<4>(ea, m, n, v0, v1);
       }
     }
   }
 }
 
 // ----------------------------------------------------------------------------- epilogues
+// Every epilogue handles W (4 or 8) consecutive columns n..n+W-1 of one output row m; v0/v1 are
+// the fp32 accumulators of the first/second accumulator set.
 
+template <typename T, int W>
+struct PackW;
 template <typename T>
-__device__ __forceinline__ void store4(T* p, f32x4 v) {
-  typename Traits<T>::vec4 o;
+struct PackW<T, 4> { typedef typename Traits<T>::vec4 type; };
+template <typename T>
+struct PackW<T, 8> { typedef typename Traits<T>::vec8 type; };
+
+template <typename T, int W>
+__device__ __forceinline__ void store_w(T* p, const float* v) {
+  typename PackW<T, W>::type o;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) o[r] = Traits<T>::from_f32(v[r]);
-  *(typename Traits<T>::vec4*)p = o;
+  for (int r = 0; r < W; ++r) o[r] = Traits<T>::from_f32(v[r]);
+  *(typename PackW<T, W>::type*)p = o;
 }
-template <typename T>
-__device__ __forceinline__ f32x4 load4(const T* p) {
-  typename Traits<T>::vec4 o = *(const typename Traits<T>::vec4*)p;
-  f32x4 v;
+template <typename T, int W>
+__device__ __forceinline__ void load_w(const T* p, float* v) {
+  typename PackW<T, W>::type o = *(const typename PackW<T, W>::type*)p;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) v[r] = Traits<T>::to_f32(o[r]);
-  return v;
+  for (int r = 0; r < W; ++r) v[r] = Traits<T>::to_f32(o[r]);
+}
+template <typename T, int W>
+__device__ __forceinline__ void add_w(const T* p, float* v) {
+  float t[W];
+  load_w<T, W>(p, t);
+#pragma unroll
+  for (int r = 0; r < W; ++r) v[r] += t[r];
+}
+template <int W>
+__device__ __forceinline__ void keep_w(const DropoutParams& d, size_t e, bool* keep) {
+#pragma unroll
+  for (int q = 0; q < W / 4; ++q) dropout_keep4(d, (e >> 2) + q, keep + 4 * q);
 }
 
 // out = acc (+ bias[n])
@@ -261,9 +280,10 @@ struct EpiStore {
     const T* bias;  // nullable
     int ldc;
   };
-  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 v, f32x4) {
-    if (a.bias) v += load4<T>(a.bias + n);
-    store4<T>(a.out + (size_t)m * a.ldc + n, v);
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float*) {
+    if (a.bias) add_w<T, W>(a.bias + n, v);
+    store_w<T, W>(a.out + (size_t)m * a.ldc + n, v);
   }
 };
 
@@ -280,53 +300,59 @@ struct EpiGateUp {
     int ldc;
     DropoutParams drop;
   };
-  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 g, f32x4 u) {
-    if (a.b_gate) g += load4<T>(a.b_gate + n);
-    if (a.b_up) u += load4<T>(a.b_up + n);
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* g, float* u) {
+    if (a.b_gate) add_w<T, W>(a.b_gate + n, g);
+    if (a.b_up) add_w<T, W>(a.b_up + n, u);
     size_t e = (size_t)m * a.ldc + n;
-    f32x4 h;
+    float h[W];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) h[r] = silu_f32(g[r]) * u[r];
+    for (int r = 0; r < W; ++r) h[r] = silu_f32(g[r]) * u[r];
     if (a.drop.enabled) {
-      bool keep[4];
-      dropout_keep4(a.drop, e >> 2, keep);
+      bool keep[W];
+      keep_w<W>(a.drop, e, keep);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
+      for (int r = 0; r < W; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
       if (a.mask_out) {
-        uint32_t packed = 0;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) packed |= (keep[r] ? 1u : 0u) << (8 * r);
-        *(uint32_t*)(a.mask_out + e) = packed;
+        for (int q = 0; q < W / 4; ++q) {
+          uint32_t packed = 0;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) packed |= (keep[4 * q + r] ? 1u : 0u) << (8 * r);
+          *(uint32_t*)(a.mask_out + e + 4 * q) = packed;
+        }
       }
     } else if (a.mask_out) {
-      *(uint32_t*)(a.mask_out + e) = 0x01010101u;
+#pragma unroll
+      for (int q = 0; q < W / 4; ++q) *(uint32_t*)(a.mask_out + e + 4 * q) = 0x01010101u;
     }
-    store4<T>(a.h + e, h);
-    if (a.g_save) store4<T>(a.g_save + e, g);
-    if (a.u_save) store4<T>(a.u_save + e, u);
+    store_w<T, W>(a.h + e, h);
+    if (a.g_save) store_w<T, W>(a.g_save + e, g);
+    if (a.u_save) store_w<T, W>(a.u_save + e, u);
   }
 };
 
-// Gating backward on 4 consecutive elements: dA = dH*keep/(1-p); dU = dA*silu(G); dG = dA*U*silu'(G)
-template <typename T>
-__device__ __forceinline__ void gating_bwd4(const DropoutParams& drop, size_t e, f32x4 dh,
-                                            const T* g, const T* u, T* dg, T* du) {
-  f32x4 gv = load4<T>(g + e), uv = load4<T>(u + e);
+// Gating backward on W consecutive elements: dA = dH*keep/(1-p); dU = dA*silu(G); dG = dA*U*silu'(G)
+template <typename T, int W>
+__device__ __forceinline__ void gating_bwd_w(const DropoutParams& drop, size_t e, float* dh,
+                                             const T* g, const T* u, T* dg, T* du) {
+  float gv[W], uv[W], dgv[W], duv[W];
+  load_w<T, W>(g + e, gv);
+  load_w<T, W>(u + e, uv);
   if (drop.enabled) {
-    bool keep[4];
-    dropout_keep4(drop, e >> 2, keep);
+    bool keep[W];
+    keep_w<W>(drop, e, keep);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) dh[r] = keep[r] ? dh[r] * drop.scale : 0.f;
+    for (int r = 0; r < W; ++r) dh[r] = keep[r] ? dh[r] * drop.scale : 0.f;
   }
-  f32x4 dgv, duv;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+  for (int r = 0; r < W; ++r) {
     float s = sigmoid_f32(gv[r]);
     duv[r] = dh[r] * (gv[r] * s);
     dgv[r] = dh[r] * uv[r] * (s * (1.0f + gv[r] * (1.0f - s)));
   }
-  store4<T>(dg + e, dgv);
-  store4<T>(du + e, duv);
+  store_w<T, W>(dg + e, dgv);
+  store_w<T, W>(du + e, duv);
 }
 
 template <typename T>
@@ -339,8 +365,9 @@ struct EpiDh {
     int ldc;
     DropoutParams drop;
   };
-  static __device__ __forceinline__ void apply(const Args& a, int m, int n, f32x4 dh, f32x4) {
-    gating_bwd4<T>(a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*) {
+    gating_bwd_w<T, W>(a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
   }
 };
 

@@ -1,6 +1,12 @@
 // One translation unit per (dtype, GEMM kind): compiled with -DGMLP_DT=<0|1> -DGMLP_KIND=<0..4>
 // so the kernels build in parallel.  Each unit instantiates the LARGE and MEDIUM tile classes.
+#include "gemm_v2.hpp"
 #include "launch.hpp"
+
+#ifndef GMLP_V2_BK
+#define GMLP_V2_BK 64  // reduction elements per LDS ring slot
+#define GMLP_V2_NS 2   // ring depth
+#endif
 
 namespace gmlp {
 
@@ -12,6 +18,8 @@ typedef bf16 DT;
 
 #define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
   if (tile_class == TILE_LARGE)                                                                  \
+    return launch_gemm_v2<DT, 256, BN_L, GMLP_V2_BK, GMLP_V2_NS, 2, 2, AKS, BKS, NB, EPI<DT>>(ga, ea, s); \
+  if (tile_class == TILE_LARGE_V1)                                                               \
     return launch_gemm<DT, 256, BN_L, 64, 2, 2, AKS, BKS, NB, false, EPI<DT>>(ga, ea, s);         \
   return launch_gemm<DT, 128, BN_M, 64, 2, 2, AKS, BKS, NB, true, EPI<DT>>(ga, ea, s);
 

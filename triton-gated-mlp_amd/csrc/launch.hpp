@@ -6,7 +6,7 @@ namespace gmlp {
 
 // Tile classes.  LARGE: 256x256x64 output tiles, 4 wavefronts of 128x128 (full tiles only).
 // MEDIUM: 128x128x64, 4 wavefronts of 64x64, with edge predication (any M, N%8, K%8).
-enum TileClass { TILE_LARGE = 0, TILE_MEDIUM = 1 };
+enum TileClass { TILE_LARGE = 0, TILE_MEDIUM = 1, TILE_LARGE_V1 = 2 };
 
 // kinds of GEMM the gated MLP needs; each is instantiated per dtype and tile class.
 template <typename T>
