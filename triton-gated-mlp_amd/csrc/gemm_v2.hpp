@@ -25,15 +25,27 @@ namespace gmlp {
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) void lds_void;
-typedef __amdgpu_buffer_rsrc_t buffer_rsrc;
+typedef int buffer_rsrc __attribute__((ext_vector_type(4)));
 
+// Raw buffer descriptor over the whole address range behind `base` (offsets are 32-bit bytes).
 __device__ __forceinline__ buffer_rsrc make_rsrc(const void* base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
+  uint64_t b = (uint64_t)base;
+  buffer_rsrc r = {(int)(uint32_t)b, (int)((b >> 32) & 0xffffu), 0x7FFFFFFF, 0x00020000};
+  return r;
 }
-// 16 bytes per lane from (rsrc base + soffset + voffset) to LDS at (lds_wave_base + 16*lane).
+// 16 bytes per lane from (rsrc base + soffset + voffset) to LDS byte address (lds_wave_base +
+// 16*lane).  Written as assembly on purpose: the compiler's bookkeeping for the LDS-DMA builtins
+// makes every later LDS read it cannot disambiguate (the transpose reads) wait for ALL loads in
+// flight; here the ordering is explicit instead (wait_vmem + barrier before a slot is read).
 __device__ __forceinline__ void load16_to_lds(buffer_rsrc r, uint32_t voffset, uint32_t soffset,
-                                              void* lds_wave_base) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)lds_wave_base, 16, voffset, soffset, 0, 0);
+                                              uint32_t lds_wave_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_wave_base), "v"(voffset), "s"(r), "s"(soffset)
+      : "memory");
 }
 
 // The LDS write of a global->LDS load is complete when the wavefront's vector-memory counter has
@@ -81,15 +93,6 @@ struct TileV2 {
     }
   }
 
-  // Issue this wavefront's share of the tile whose origin is at byte `origin` of the buffer.
-  static __device__ __forceinline__ void issue(buffer_rsrc r, uint32_t origin,
-                                               const uint32_t (&off)[PER_WAVE], char* lds_tile,
-                                               int wave) {
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; ++i)
-      load16_to_lds(r, off[i], origin, lds_tile + (wave * PER_WAVE + i) * 1024);
-  }
-
   // MFMA fragment (8 reduction elements per lane) for rows row0..row0+31, reduction step ks.
   static __device__ __forceinline__ vec8 frag(const char* lds_tile, int row0, int ks, int lane) {
     if (!KS) {
@@ -134,10 +137,15 @@ struct ConfigV2 {
   static_assert((NS - 1) * LOADS < 64, "vmcnt is a 6-bit counter");
 };
 
+#ifndef GMLP_V2_LOAD_STRIDE
+#define GMLP_V2_LOAD_STRIDE 2
+#endif
+
 template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
           int NB, typename Epi>
 __global__ void __launch_bounds__(WGM* WGN * 64)
     gemm_kernel_v2(GemmArgs ga, typename Epi::Args ea) {
+  constexpr int LOAD_STRIDE = GMLP_V2_LOAD_STRIDE;
   typedef ConfigV2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB> Cfg;
   typedef typename Cfg::ATile ATile;
   typedef typename Cfg::BTile BTile;
@@ -182,6 +190,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
   const uint32_t b_step = B_KS ? (uint32_t)BK * ga.ldb * 2 : (uint32_t)BK * 2;
   const uint32_t a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
   const uint32_t b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem;
   const buffer_rsrc ra[2] = {make_rsrc(ga.A[0]), make_rsrc(ga.A[1])};
   const buffer_rsrc rb[2] = {make_rsrc(ga.B[0]), make_rsrc(ga.B[1])};
 
@@ -192,7 +201,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
     int kt = kt_req < kt_total ? kt_req : kt_total - 1;
     int seg = kt >= kt_seg ? 1 : 0;
     int kk = kt - seg * kt_seg;
-    char* s = smem + (kt_req & (NS - 1)) * STAGE;
+    uint32_t s = lds_base + (kt_req & (NS - 1)) * STAGE;
     if (x < ATile::PER_WAVE) {
       load16_to_lds(seg ? ra[1] : ra[0], aoff[x], a_org + kk * a_step,
                     s + (wave * ATile::PER_WAVE + x) * 1024);
@@ -226,47 +235,55 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
   // share of the global->LDS loads of a tile}, and the scheduler is told to keep the slots.
   constexpr int NMFMA = NB * TM * TN;
   static_assert(NFRAG < NMFMA, "operand reads must fit in the MFMA slots");
-  constexpr int LPS = (L + (NMFMA - NFRAG) - 1) / (NMFMA - NFRAG);  // loads per slot
-  auto step = [&](int buf, auto frags_c, int fkt, int fks, auto loads_c, int lkt) __attribute__((always_inline)) {
+  // The refill of a ring slot starts in the step that retires it and is paced at one load per
+  // LOAD_STRIDE slots (the vector-memory front end takes a 1 KiB wavefront load every ~16 cycles
+  // for the whole CU; issuing faster blocks the wavefront, and the MFMAs queued behind it).
+  // g0 = slot number of this step's first MFMA, counted from the retiring step's first slot.
+  static_assert(L * LOAD_STRIDE <= KSTEPS * NMFMA, "a tile's loads must fit in one tile of slots");
+  auto step = [&](int buf, auto frags_c, int fkt, int fks, auto loads_c, int g0, int lkt) __attribute__((always_inline)) {
     constexpr bool FRAGS = decltype(frags_c)::value, LOADS = decltype(loads_c)::value;
 #pragma unroll
     for (int q = 0; q < NMFMA; ++q) {
       const int b = q / (TN * TM), j = (q / TM) % TN, i = q % TM;
       acc[b][i][j] = Traits<T>::mfma(bf[buf][b][j], af[buf][i], acc[b][i][j]);
       if (FRAGS && q < NFRAG) load_frag(buf ^ 1, fkt, fks, q);
-      if (LOADS && q >= NFRAG) {
-#pragma unroll
-        for (int x = (q - NFRAG) * LPS; x < (q - NFRAG + 1) * LPS && x < L; ++x) issue_one(lkt, x);
-      }
+      const int g = g0 + q;
+      if (LOADS && g % LOAD_STRIDE == 0 && g / LOAD_STRIDE < L) issue_one(lkt, g / LOAD_STRIDE);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
   // One reduction tile kt (ring slot kt % NS).  NEXT: tile kt+1 exists; then this tile's last step
   // retires the slot: wait until tile kt+1 has landed (the NS-2 younger tiles stay in flight),
-  // barrier, and refill the slot with tile kt+NS while reading tile kt+1's first operands.
+  // barrier, start refilling the slot with tile kt+NS and read tile kt+1's first operands.  The
+  // earlier steps carry the rest of the refill that tile kt-1's retirement started.
   auto tile_body = [&](int kt, auto next_c) __attribute__((always_inline)) {
     constexpr bool NEXT = decltype(next_c)::value;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const int buf = (KSTEPS & 1) ? ((kt + ks) & 1) : (ks & 1);
       if (ks < KSTEPS - 1) {
-        step(buf, std::true_type{}, kt, ks + 1, std::false_type{}, 0);
+        step(buf, std::true_type{}, kt, ks + 1, std::integral_constant<bool, NEXT>{}, (ks + 1) * NMFMA,
+             kt - 1 + NS);
       } else if (NEXT) {
         wait_vmem<(NS - 2) * L>();
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        step(buf, std::true_type{}, kt + 1, 0, std::true_type{}, kt + NS);
+        step(buf, std::true_type{}, kt + 1, 0, std::true_type{}, 0, kt + NS);
       } else {
-        step(buf, std::false_type{}, 0, 0, std::false_type{}, 0);
+        step(buf, std::false_type{}, 0, 0, std::false_type{}, 0, 0);
       }
     }
   };
 
-  // Prologue: fill the ring with tiles 0 .. NS-1, wait for tile 0.
+  // Prologue: tiles 0 .. NS-2 entirely, and of tile NS-1 the loads a retiring step would issue
+  // (tile 0's first steps issue the rest); wait for tile 0.
+  constexpr int L_HEAD = (NMFMA + LOAD_STRIDE - 1) / LOAD_STRIDE < L ? (NMFMA + LOAD_STRIDE - 1) / LOAD_STRIDE : L;
 #pragma unroll
-  for (int p = 0; p < NS; ++p) issue_tile(p);
-  wait_vmem<(NS - 1) * L>();
+  for (int p = 0; p < NS - 1; ++p) issue_tile(p);
+#pragma unroll
+  for (int x = 0; x < L_HEAD; ++x) issue_one(NS - 1, x);
+  wait_vmem<(NS - 2) * L + L_HEAD>();
   __syncthreads();
 #pragma unroll
   for (int f = 0; f < NFRAG; ++f) load_frag(0, 0, 0, f);
