@@ -200,6 +200,8 @@ __global__ void __launch_bounds__(DEC_SPLIT * 64)
 template <typename T>
 hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
                          const T* bu, const T* bd, T* h, T* y, int M, int K, int N, hipStream_t s) {
+  if (decode_stream_supported(M, K, N))
+    return launch_decode_stream<T>(x, wg, wu, wd, bg, bu, bd, h, y, M, K, N, s);
   int nblocks = N / 16;
   hipLaunchKernelGGL(decode_gateup_kernel<T>, dim3((nblocks + 3) / 4), dim3(256), 0, s, x, wg, wu,
                      bg, bu, h, M, K, N);

@@ -1,0 +1,267 @@
+// Skinny-M (M <= 16) weight-streaming kernels, HBM-bound: every weight byte is fetched once, in
+// 512-byte row segments moved global -> LDS without passing through registers.
+//
+// One persistent workgroup of three wavefronts per CU.  The workgroup owns blocks of 2 x 16 weight
+// rows (rb = blockIdx.x, blockIdx.x + gridDim.x, ...) that share one set of token operands: rows
+// r..r+15 of W_gate and of W_up (GATED), or 32 consecutive rows of W_down; its wavefronts split the reduction range in
+// near-equal runs of 256-element chunks and combine their partial sums through LDS at the
+// end of each block (fixed order, so the result is deterministic).  Each wavefront runs a private
+// ring of 3 LDS slots; a slot holds one stage = 256 reduction elements of the 16 weight rows of
+// each matrix.  The matching token-row operands (x or H, L2-resident) are fetched straight into
+// registers, three stages ahead as well.  Achieved HBM bandwidth follows the bytes in flight per
+// CU, and LDS capacity bounds those: wavefronts x 3 slots x slot size fill 144 of the 160 KiB.
+// The stream of stages runs on across block boundaries, so the ring never drains; loads past the
+// end re-fetch the last stage into a free slot, which keeps the in-flight count constant.
+//
+//   GATED:   H[m, r] = silu(x.W_gate[r] + b_gate[r]) * (x.W_up[r] + b_up[r])     (r over N)
+//   !GATED:  Y[m, r] = H.W_down[r] + b_down[r]                                   (r over K)
+//
+// LDS layout of a slot: 2 regions of 16 rows x 512 bytes; the 16-byte chunk c of row r is
+// stored at position c ^ r, so the 16 lanes that read one chunk index of 16 different rows for
+// v_mfma_f32_16x16x32 hit 16 different bank groups.
+//
+// All vector-memory loads of the main loop are written as assembly and ordered by explicit
+// s_waitcnt vmcnt(N): the compiler does not see them, so it cannot serialise them either.
+#include "launch.hpp"
+#include "lds_dma.hpp"
+
+namespace gmlp {
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Mfma16x;
+template <>
+struct Mfma16x<f16> {
+  static __device__ __forceinline__ f32x4v run(f16x8 a, f16x8 b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16x<bf16> {
+  static __device__ __forceinline__ f32x4v run(bf16x8 a, bf16x8 b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int DS_CH = 256;            // reduction elements per stage
+constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
+constexpr int DS_RD = 3;              // ring slots per wavefront (and stages in flight)
+constexpr int DS_WAVES = 3;           // wavefronts per workgroup
+
+struct StreamArgs {
+  const void* x;      // [M, ldx] token rows (x or H)
+  const void* w[2];   // [R, red] weight matrices
+  const void* bias[2];
+  void* out;          // [M, ldo]
+  int M, R, red, ldx, ldo;
+};
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane into registers; completion is tracked by the caller (wait_vmem_keep).
+__device__ __forceinline__ i32x4 load16_async(buffer_rsrc r, uint32_t voffset, uint32_t soffset) {
+  i32x4 v;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
+               : "=v"(v)
+               : "v"(voffset), "s"(r), "s"(soffset)
+               : "memory");
+  return v;
+}
+// s_waitcnt vmcnt(N) that also "defines" the 8 registers a stage's token operands arrive in, so
+// no use of them can be scheduled above the wait.
+template <int N>
+__device__ __forceinline__ void wait_vmem_keep(i32x4 (&x)[8]) {
+  asm volatile("s_waitcnt vmcnt(%8)"
+               : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]),
+                 "+v"(x[7])
+               : "n"(N)
+               : "memory");
+}
+
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs a) {
+  typedef typename Traits<T>::vec8 vec8;
+  constexpr int NMAT = 2;                       // 16-row regions per stage
+  constexpr int BLOCK_ROWS = GATED ? 16 : 32;   // weight rows (per matrix) a block advances by
+  constexpr int SLOT = NMAT * DS_REGION;
+  constexpr int LPS = 8 + 8 * NMAT;  // load instructions per stage (token operands + weights)
+  static_assert((DS_RD - 1) * LPS < 64, "the younger stages must fit the 6-bit vmcnt");
+
+  extern __shared__ __align__(1024) char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem + wave * (DS_RD * SLOT);
+  char* ring = smem + wave * (DS_RD * SLOT);
+  float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [2 parities][waves-1][NMAT][64][4]
+
+  const int nblocks = a.R / BLOCK_ROWS;
+  const int chunks = a.red / DS_CH;
+  // wavefront w reduces chunks [c0, c0 + spb)
+  const int c0 = (chunks * wave) / DS_WAVES;
+  const int spb = (chunks * (wave + 1)) / DS_WAVES - c0;
+  const int my_blocks = (nblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int total = my_blocks * spb;
+
+  // Per-lane byte offsets: weights, 8 load instructions per region (2 rows x 512 bytes each);
+  // token operands, the 16 bytes of row lane%16 this lane feeds to each of the stage's 8 MFMAs.
+  const int r16 = lane & 15, kg = lane >> 4;
+  uint32_t woff[8], xoff;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    int row = 2 * q + (lane >> 5), pos = lane & 31;
+    woff[q] = (uint32_t)(row * a.red + (pos ^ row) * 8) * 2u;
+  }
+  {
+    int xr = r16 < a.M ? r16 : a.M - 1;  // rows past M repeat the last token row (never stored)
+    xoff = (uint32_t)(xr * a.ldx + kg * 8) * 2u;
+  }
+  const buffer_rsrc rx = make_rsrc(a.x);
+  const buffer_rsrc rw[2] = {make_rsrc(a.w[0]), make_rsrc(a.w[1])};
+
+  i32x4 xf[DS_RD][8];
+
+  // Stage i_req of this wavefront's stream: token operands into xf[u], weights into ring slot u.
+  auto issue_stage = [&](int i_req, int u) __attribute__((always_inline)) {
+    int i = i_req < total ? i_req : total - 1;
+    int j = i / spb, c = i - j * spb;
+    int rb = (int)blockIdx.x + j * (int)gridDim.x;
+    uint32_t koff = (uint32_t)((c0 + c) * DS_CH) * 2u;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) xf[u][q] = load16_async(rx, xoff, koff + q * 64);
+    uint32_t slot = lds_base + (uint32_t)u * SLOT;
+    uint32_t woffs = (uint32_t)rb * (uint32_t)BLOCK_ROWS * (uint32_t)a.red * 2u + koff;
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        load16_to_lds<true>(rw[m], woff[q], woffs, slot + m * DS_REGION + q * 1024);
+  };
+
+  f32x4v acc[NMAT];
+#pragma unroll
+  for (int m = 0; m < NMAT; ++m) acc[m] = f32x4v{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int p = 0; p < DS_RD; ++p) issue_stage(p, p);
+
+  int in_block = 0, blk = 0;
+  for (int i0 = 0; i0 < total; i0 += DS_RD) {
+#pragma unroll
+    for (int u = 0; u < DS_RD; ++u) {
+      const int i = i0 + u;
+      if (i < total) {
+        wait_vmem_keep<(DS_RD - 1) * LPS>(xf[u]);
+        const char* slot = ring + u * SLOT;
+#pragma unroll
+        for (int ks = 0; ks < DS_CH / 32; ++ks) {
+          int pos = ((ks * 4 + kg) ^ r16) << 4;
+          vec8 xv = __builtin_bit_cast(vec8, xf[u][ks]);
+#pragma unroll
+          for (int m = 0; m < NMAT; ++m) {
+            vec8 wf = *(const vec8*)(slot + m * DS_REGION + r16 * 512 + pos);
+            acc[m] = Mfma16x<T>::run(wf, xv, acc[m]);
+          }
+        }
+        // The MFMAs above consumed every LDS read of this slot, so it can be refilled.
+        issue_stage(i + DS_RD, u);
+
+        if (++in_block == spb) {
+          // Block finished: wavefronts 1.. hand their partial sums to wavefront 0.  A lane holds
+          // token row m = lane%16 and, per region, weight rows 4*(lane/16) + r of the block.
+          in_block = 0;
+          float* pp = part + (blk & 1) * ((DS_WAVES - 1) * NMAT * 256);
+          if (wave > 0) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+              *(f32x4v*)(pp + ((wave - 1) * NMAT + m) * 256 + lane * 4) = acc[m];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+          if (wave == 0 && r16 < a.M) {
+            int rb = (int)blockIdx.x + blk * (int)gridDim.x;
+            int r0 = rb * BLOCK_ROWS + 4 * kg;
+            float v[NMAT][4];
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[m][r] = acc[m][r];
+#pragma unroll
+              for (int w = 0; w < DS_WAVES - 1; ++w) {
+                f32x4v o = *(const f32x4v*)(pp + (w * NMAT + m) * 256 + lane * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[m][r] += o[r];
+              }
+              if (a.bias[m]) add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
+            }
+            if (GATED) {
+              float res[4];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) res[r] = silu_f32(v[0][r]) * v[1][r];
+              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
+            } else {
+              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, v[0]);
+              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16, v[1]);
+            }
+          }
+#pragma unroll
+          for (int m = 0; m < NMAT; ++m) acc[m] = f32x4v{0.f, 0.f, 0.f, 0.f};
+          ++blk;
+        }
+      }
+    }
+  }
+  wait_vmem<0>();
+}
+
+template <typename T, bool GATED>
+static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
+  constexpr int LDS = DS_WAVES * DS_RD * 2 * DS_REGION + 2 * (DS_WAVES - 1) * 2 * 256 * 4;
+  auto kern = decode_stream_kernel<T, GATED>;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int nblocks = a.R / (GATED ? 16 : 32);
+  int grid = nblocks < num_cu ? nblocks : num_cu;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);
+  return hipGetLastError();
+}
+
+bool decode_stream_supported(int M, int K, int N) {
+  return M >= 1 && M <= 16 && K % DS_CH == 0 && N % DS_CH == 0 && K >= DS_WAVES * DS_CH && N >= DS_WAVES * DS_CH &&
+         (int64_t)K * N * 2 < ((int64_t)1 << 31);
+}
+
+template <typename T>
+hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
+                                const T* bu, const T* bd, T* h, T* y, int M, int K, int N,
+                                hipStream_t s) {
+  static int num_cu = 0;
+  if (num_cu == 0) {
+    int dev = 0, n = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    num_cu = n > 0 ? n : 256;
+  }
+  StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N};
+  hipError_t e = launch_stream<T, true>(a1, num_cu, s);
+  if (e != hipSuccess) return e;
+  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K};
+  return launch_stream<T, false>(a2, num_cu, s);
+}
+
+template hipError_t launch_decode_stream<f16>(const f16*, const f16*, const f16*, const f16*,
+                                              const f16*, const f16*, const f16*, f16*, f16*, int,
+                                              int, int, hipStream_t);
+template hipError_t launch_decode_stream<bf16>(const bf16*, const bf16*, const bf16*, const bf16*,
+                                               const bf16*, const bf16*, const bf16*, bf16*, bf16*,
+                                               int, int, int, hipStream_t);
+
+}  // namespace gmlp

@@ -1,0 +1,53 @@
+// Global -> LDS transfers that bypass the vector registers (buffer_load ... lds) and the explicit
+// vector-memory waits that order them, shared by the GEMM and the skinny-M streaming kernels.
+#pragma once
+#include "common.hpp"
+
+namespace gmlp {
+
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) void lds_void;
+typedef int buffer_rsrc __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor over the whole address range behind `base` (offsets are 32-bit bytes).
+__device__ __forceinline__ buffer_rsrc make_rsrc(const void* base) {
+  uint64_t b = (uint64_t)base;
+  buffer_rsrc r = {(int)(uint32_t)b, (int)((b >> 32) & 0xffffu), 0x7FFFFFFF, 0x00020000};
+  return r;
+}
+// 16 bytes per lane from (rsrc base + soffset + voffset) to LDS byte address (lds_wave_base +
+// 16*lane).  Written as assembly on purpose: the compiler's bookkeeping for the LDS-DMA builtins
+// makes every later LDS read it cannot disambiguate (the transpose reads) wait for ALL loads in
+// flight; here the ordering is explicit instead (wait_vmem + barrier before a slot is read).
+// STREAM marks data that is read once (non-temporal: do not keep it in the caches).
+template <bool STREAM = false>
+__device__ __forceinline__ void load16_to_lds(buffer_rsrc r, uint32_t voffset, uint32_t soffset,
+                                              uint32_t lds_wave_base) {
+  if (STREAM) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen nt lds"
+        :
+        : "s"(lds_wave_base), "v"(voffset), "s"(r), "s"(soffset)
+        : "memory");
+  } else {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen lds"
+        :
+        : "s"(lds_wave_base), "v"(voffset), "s"(r), "s"(soffset)
+        : "memory");
+  }
+}
+
+// The LDS write of a global->LDS load is complete when the wavefront's vector-memory counter has
+// drained past it; a workgroup barrier alone does not wait for it.  N = loads allowed in flight.
+template <int N>
+__device__ __forceinline__ void wait_vmem() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+}  // namespace gmlp
