@@ -122,7 +122,7 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
  * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch is [M,N] in dtype;
  * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
  * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
- * Requires K % 512 == 0 and N % 512 == 0.
+ * Requires K % 32 == 0 and N % 256 == 0 (the LDS-ring streaming kernels run when K % 256 == 0 too).
  */
 int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                     const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
