@@ -31,6 +31,8 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
 M, K, N = 8192, 4096, 14336
 DTYPE = torch.float16
+# rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain copy of known size reads) + WRITE_SIZE, per launch
+GATEUP_TRAFFIC_BYTES = 3.525e9
 
 
 def _median(v):
@@ -151,6 +153,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip per-kernel breakdown and decode line")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -158,6 +162,13 @@ def main():
         sys.exit("bench.py needs an AMD GPU (no CPU fallback for the fused path)")
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+
+    if args.calibration_copy:
+        src = torch.ones(256 * 1024 * 1024, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     mlp, x, dY = _make_module(dev)
     params = list(mlp.parameters())
@@ -191,7 +202,9 @@ def main():
     roofline = {"kernel": "gemm_kernel<f16,256,128,64,...,EpiGateUp> (gate/up forward GEMM + SiLU-gating epilogue)",
                 "bound": "mfma", "achieved": round(dom_flop / avg / 1e9, 1), "peak": PEAK_MFMA_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_flop / avg / 1e9 / PEAK_MFMA_F16_TFLOPS, 4),
-                "avg_launch_ms": round(avg, 4), "flop_per_launch": dom_flop, "traffic": None}
+                "avg_launch_ms": round(avg, 4), "flop_per_launch": dom_flop, "traffic": GATEUP_TRAFFIC_BYTES,
+                "traffic_note": "HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                "(profiles/gateup_gemm_hbm_traffic.txt); algorithmic bytes are 1.007e9"}
 
     line = {
         "metric": "fwd+bwd TFLOP/s & % MFMA peak, fp16 M=8192 K=4096 N=14336 (1 GPU)",
