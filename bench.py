@@ -86,9 +86,7 @@ def _kernel_breakdown(mlp, x, dY, reps):
         ("down_fwd", lambda: F.linear_fwd(hs.hidden, Wd), mnk2),
         ("dh_bwd", lambda: B.dh_bwd(dY, Wd, hs.gate, hs.up), mnk2),
         ("dx_bwd", lambda: B.dx_bwd(dg, du, Wg, Wu), 2 * mnk2),
-        ("dw_gate", lambda: B.dw_bwd(dg, xd), mnk2),
-        ("dw_up", lambda: B.dw_bwd(du, xd), mnk2),
-        ("dw_down", lambda: B.dw_bwd(dY, hs.hidden), mnk2),
+        ("dw_gate_up_down_grouped", lambda: B.dw_bwd_grouped([(dg, xd), (du, xd), (dY, hs.hidden)]), 3 * mnk2),
     ]
     out = {}
     for name, fn, flop in launches:

@@ -109,6 +109,16 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
                 int dtype, void* stream);
 
 /*
+ * Up to 3 weight gradients that share the reduction length Mred, enqueued as ONE grid when every
+ * problem fits the full-tile kernel (otherwise as `count` separate launches):
+ *   dw[i][R[i],C[i]] = lhs[i][Mred,R[i]]ᵀ · rhs[i][Mred,C[i]],  i < count.
+ * Same reference counterparts as gmlp_dw_bwd; one launch for dW_gate, dW_up and dW_down avoids
+ * three partially filled last rounds of workgroups.
+ */
+int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rhs, void* const* dw,
+                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* stream);
+
+/*
  * Bias gradient: out[C] = Σ_m a[m,C], fp32 accumulation in a fixed order (deterministic).
  * workspace: gmlp_workspace_bytes(GMLP_OP_COLSUM, M, 0, C, dtype) bytes.
  * The reference returns None for bias gradients (gated_mlp.py:200); EagerGatedMLP's autograd

@@ -252,12 +252,32 @@ def test_full_size_properties_cfg3_linearity_and_zero():
     assert not z.hidden.any()
 
 
+def test_grouped_weight_gradients_equal_single_launches():
+    """gmlp_dw_bwd_grouped (one grid) is bit-identical to three gmlp_dw_bwd launches."""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(9)
+    for M, K, N in [(2048, 2048, 5632), (512, 256, 520)]:  # full-tile class and predicated class
+        x = torch.randn(M, K, generator=g).half().to(dev)
+        dg = torch.randn(M, N, generator=g).half().to(dev)
+        du = torch.randn(M, N, generator=g).half().to(dev)
+        dy = torch.randn(M, K, generator=g).half().to(dev)
+        h = torch.randn(M, N, generator=g).half().to(dev)
+        pairs = [(dg, x), (du, x), (dy, h)]
+        grouped = ops_bwd.dw_bwd_grouped(pairs)
+        for (a, b), got in zip(pairs, grouped):
+            assert torch.equal(got, ops_bwd.dw_bwd(a, b))
+        _close("dW_gate grouped", grouped[0], dg.float().cpu().T @ x.float().cpu(), atol=ATOL * 40)
+
+
 def test_decode_matches_general_path():
     from triton_gated_mlp.ops import fwd as ops_fwd
 
     dev = _dev()
     g = torch.Generator().manual_seed(2)
-    for M, K, N, bias in [(16, 1024, 2048, True), (3, 256, 512, False), (1, 4096, 11008, True)]:
+    for M, K, N, bias in [(16, 1024, 2048, True), (3, 256, 512, False), (1, 4096, 11008, True), (5, 768, 1792, True),
+                          (16, 4096, 11008, False)]:
         x = torch.randn(M, K, generator=g).half().to(dev)
         Wg = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
         Wu = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)

@@ -270,6 +270,56 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   return hip_result(__func__, e);
 }
 
+int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rhs, void* const* dw,
+                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* stream) {
+  using namespace gmlp;
+  if (count < 1 || count > GEMM_GROUP_MAX)
+    return fail(GMLP_EINVAL, "%s: count = %d must be in 1..%d", __func__, count, GEMM_GROUP_MAX);
+  GMLP_REQUIRE_PTR(lhs); GMLP_REQUIRE_PTR(rhs); GMLP_REQUIRE_PTR(dw); GMLP_REQUIRE_PTR(R);
+  GMLP_REQUIRE_PTR(C);
+  GMLP_REQUIRE_DTYPE(dtype);
+  bool large = true;
+  for (int i = 0; i < count; ++i) {
+    GMLP_REQUIRE_PTR(lhs[i]); GMLP_REQUIRE_PTR(rhs[i]); GMLP_REQUIRE_PTR(dw[i]);
+    if (int rc = check_dims(__func__, Mred, R[i], C[i])) return rc;
+    if (int rc = check_mult8(__func__, "R", R[i])) return rc;
+    if (int rc = check_mult8(__func__, "C", C[i])) return rc;
+    GMLP_REQUIRE_ALIGNED(lhs[i]); GMLP_REQUIRE_ALIGNED(rhs[i]); GMLP_REQUIRE_ALIGNED(dw[i]);
+    large = large && pick_tile(R[i], C[i], Mred, 256) == TILE_LARGE;
+  }
+  if (!large) {
+    for (int i = 0; i < count; ++i)
+      if (int rc = gmlp_dw_bwd(lhs[i], rhs[i], dw[i], Mred, R[i], C[i], dtype, stream)) return rc;
+    return GMLP_OK;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  auto fill = [&](GemmArgs& ga, int i) {
+    ga = GemmArgs{};
+    ga.A[0] = lhs[i]; ga.A[1] = lhs[i]; ga.B[0] = rhs[i]; ga.B[1] = rhs[i];
+    ga.M = (int)R[i]; ga.N = (int)C[i]; ga.K = (int)Mred; ga.lda = (int)R[i]; ga.ldb = (int)C[i];
+    ga.nseg = 1; ga.group_m = 8;
+  };
+  hipError_t e;
+  if (dtype == GMLP_F16) {
+    GemmGroup<EpiStore<f16>::Args> grp = {};
+    grp.count = count;
+    for (int i = 0; i < count; ++i) {
+      fill(grp.ga[i], i);
+      grp.ea[i] = EpiStore<f16>::Args{(f16*)dw[i], nullptr, (int)C[i]};
+    }
+    e = launch_dw_group<f16>(grp, s);
+  } else {
+    GemmGroup<EpiStore<bf16>::Args> grp = {};
+    grp.count = count;
+    for (int i = 0; i < count; ++i) {
+      fill(grp.ga[i], i);
+      grp.ea[i] = EpiStore<bf16>::Args{(bf16*)dw[i], nullptr, (int)C[i]};
+    }
+    e = launch_dw_group<bf16>(grp, s);
+  }
+  return hip_result(__func__, e);
+}
+
 int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C, int dtype,
                 void* stream) {
   using namespace gmlp;

@@ -53,6 +53,10 @@ hipError_t launch_dw<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>:
                          hipStream_t s) {
   GMLP_DISPATCH(true, true, 1, EpiStore, 256, 128)
 }
+template <>
+hipError_t launch_dw_group<DT>(GemmGroup<EpiStore<DT>::Args>& grp, hipStream_t s) {
+  return launch_gemm_group_v2<DT, 256, 256, GMLP_V2_BK, GMLP_V2_NS, 2, 2, true, true, 1, EpiStore<DT>>(grp, s);
+}
 #endif
 
 }  // namespace gmlp

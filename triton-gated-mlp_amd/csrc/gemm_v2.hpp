@@ -109,10 +109,11 @@ struct ConfigV2 {
 #define GMLP_V2_LOAD_STRIDE 2
 #endif
 
+// Body of the kernel: workgroup `pid` of the `nwg` that cover one GEMM.
 template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
           int NB, typename Epi>
-__global__ void __launch_bounds__(WGM* WGN * 64)
-    gemm_kernel_v2(GemmArgs ga, typename Epi::Args ea) {
+__device__ __forceinline__ void gemm_v2_body(const GemmArgs& ga, const typename Epi::Args& ea,
+                                             int pid, int nwg) {
   constexpr int LOAD_STRIDE = GMLP_V2_LOAD_STRIDE;
   typedef ConfigV2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB> Cfg;
   typedef typename Cfg::ATile ATile;
@@ -131,7 +132,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
 
   const int tiles_m = ga.M / BM, tiles_n = ga.N / BN;
   int tm_i, tn_i;
-  map_tile(blockIdx.x, gridDim.x, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  map_tile(pid, nwg, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
   const int m0 = tm_i * BM, n0 = tn_i * BN;
 
   f32x16 acc[NB][TM][TN];
@@ -301,6 +302,65 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
       Epi::template apply<8>(ea, m, n, v0, v1);
     }
   }
+}
+
+template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
+          int NB, typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64)
+    gemm_kernel_v2(GemmArgs ga, typename Epi::Args ea) {
+  gemm_v2_body<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB, Epi>(ga, ea, blockIdx.x, gridDim.x);
+}
+
+// Up to GEMM_GROUP_MAX independent GEMMs of one kind in a single launch: workgroups
+// [first[g], first[g+1]) belong to problem g.  One launch instead of several removes the partially
+// filled last round of workgroups of each problem.
+constexpr int GEMM_GROUP_MAX = 3;
+template <typename EpiArgs>
+struct GemmGroup {
+  GemmArgs ga[GEMM_GROUP_MAX];
+  EpiArgs ea[GEMM_GROUP_MAX];
+  int first[GEMM_GROUP_MAX + 1];
+  int count;
+};
+
+template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
+          int NB, typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64)
+    gemm_group_kernel_v2(GemmGroup<typename Epi::Args> grp) {
+  int g = 0;
+#pragma unroll
+  for (int i = 1; i < GEMM_GROUP_MAX; ++i)
+    if (i < grp.count && (int)blockIdx.x >= grp.first[i]) g = i;
+  // copy the selected problem to registers with uniform (scalar) selects
+  GemmArgs ga = grp.ga[0];
+  typename Epi::Args ea = grp.ea[0];
+#pragma unroll
+  for (int i = 1; i < GEMM_GROUP_MAX; ++i)
+    if (g == i) { ga = grp.ga[i]; ea = grp.ea[i]; }
+  gemm_v2_body<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB, Epi>(
+      ga, ea, (int)blockIdx.x - grp.first[g], grp.first[g + 1] - grp.first[g]);
+}
+
+template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
+          int NB, typename Epi>
+hipError_t launch_gemm_group_v2(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
+  typedef ConfigV2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  auto kern = gemm_group_kernel_v2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB, Epi>;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int total = 0;
+  for (int g = 0; g < grp.count; ++g) {
+    grp.first[g] = total;
+    total += (grp.ga[g].M / BM) * (grp.ga[g].N / BN);
+  }
+  for (int g = grp.count; g <= GEMM_GROUP_MAX; ++g) grp.first[g] = total;
+  hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);
+  return hipGetLastError();
 }
 
 template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,

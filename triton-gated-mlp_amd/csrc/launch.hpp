@@ -1,6 +1,7 @@
 // Host-side launch interface between the C ABI (api.hip) and the kernel translation units.
 #pragma once
 #include "gemm.hpp"
+#include "gemm_v2.hpp"
 
 namespace gmlp {
 
@@ -24,6 +25,10 @@ hipError_t launch_dx(int tile_class, const GemmArgs& ga, const typename EpiStore
 template <typename T>
 hipError_t launch_dw(int tile_class, const GemmArgs& ga, const typename EpiStore<T>::Args& ea,
                      hipStream_t s);  // A KS, B KS
+
+// Several LARGE-class weight-gradient GEMMs (every problem: whole 256x256 tiles, Mred % 64 == 0).
+template <typename T>
+hipError_t launch_dw_group(GemmGroup<typename EpiStore<T>::Args>& grp, hipStream_t s);
 
 // Generic launcher used by the instantiation units.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool B_KS, int NB,

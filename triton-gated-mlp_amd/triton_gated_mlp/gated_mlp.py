@@ -145,20 +145,24 @@ class FusedGatedMLPFullFunction(Function):
         need = ctx.needs_input_grad
         dy = dy.contiguous()
         dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
+        dw_jobs = []  # (slot, lhs, rhs): the weight gradients go out as one grouped launch
         if any(need[:5]):
             dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset)
             if need[0]:
                 dx = _bwd.dx_bwd(dg, du, W_gate, W_up)
             if need[1]:
-                dW_gate = _bwd.dw_bwd(dg, x)
+                dw_jobs.append(("gate", dg, x))
             if ctx.has_bias[0] and need[2]:
                 db_gate = _bwd.colsum(dg)
             if need[3]:
-                dW_up = _bwd.dw_bwd(du, x)
+                dw_jobs.append(("up", du, x))
             if ctx.has_bias[1] and need[4]:
                 db_up = _bwd.colsum(du)
         if need[5]:
-            dW_down = _bwd.dw_bwd(dy, hidden)
+            dw_jobs.append(("down", dy, hidden))
+        if dw_jobs:
+            grads = dict(zip([j[0] for j in dw_jobs], _bwd.dw_bwd_grouped([(j[1], j[2]) for j in dw_jobs])))
+            dW_gate, dW_up, dW_down = grads.get("gate"), grads.get("up"), grads.get("down")
         if ctx.has_bias[2] and need[6]:
             db_down = _bwd.colsum(dy)
         return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None

@@ -106,6 +106,41 @@ def dw_bwd(lhs: Tensor, rhs: Tensor) -> Tensor:
     return dw
 
 
+def dw_bwd_grouped(pairs):
+    """Weight gradients [lhs_iᵀ · rhs_i for (lhs_i, rhs_i) in pairs] (at most 3 pairs sharing the
+    reduction length) enqueued as one grid when every problem fits the full-tile kernel."""
+    import ctypes
+
+    pairs = [(_c(a), _c(b)) for a, b in pairs]
+    if not 1 <= len(pairs) <= 3:
+        raise ValueError("dw_bwd_grouped takes 1 to 3 (lhs, rhs) pairs")
+    M = pairs[0][0].shape[0]
+    for a, b in pairs:
+        if a.ndim != 2 or b.ndim != 2 or a.shape[0] != M or b.shape[0] != M:
+            raise ValueError("every pair must be 2-D with the same number of rows")
+    dev = _cabi.require_gpu(*[t for p in pairs for t in p])
+    code = _cabi.dtype_code(pairs[0][0].dtype)
+    if M == 0:
+        return [torch.zeros((a.shape[1], b.shape[1]), dtype=a.dtype, device=dev) for a, b in pairs]
+    outs = [torch.empty((a.shape[1], b.shape[1]), dtype=a.dtype, device=dev) for a, b in pairs]
+    n = len(pairs)
+    PtrArr, I64Arr = ctypes.c_void_p * n, ctypes.c_int64 * n
+    lhs = PtrArr(*[a.data_ptr() for a, _ in pairs])
+    rhs = PtrArr(*[b.data_ptr() for _, b in pairs])
+    dws = PtrArr(*[o.data_ptr() for o in outs])
+    R = I64Arr(*[a.shape[1] for a, _ in pairs])
+    C = I64Arr(*[b.shape[1] for _, b in pairs])
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_dw_bwd_grouped(
+                n, ctypes.cast(lhs, ctypes.c_void_p), ctypes.cast(rhs, ctypes.c_void_p),
+                ctypes.cast(dws, ctypes.c_void_p), M, ctypes.cast(R, ctypes.c_void_p),
+                ctypes.cast(C, ctypes.c_void_p), code, _cabi.stream_ptr(dev),
+            )
+        )
+    return outs
+
+
 def colsum(a: Tensor) -> Tensor:
     """Σ_m a[m,:] with fp32 accumulation in a fixed order (bias gradient)."""
     if a.ndim != 2:
