@@ -6,7 +6,6 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 
 #include "launch.hpp"
 
@@ -70,13 +69,15 @@ int hip_result(const char* fn, hipError_t e) {
 }
 
 // LARGE tiles need whole 256 x bn_large tiles, a reduction that is a multiple of 64, and enough
-// tiles to occupy the chip; everything else runs on the predicated MEDIUM class.
+// tiles to occupy the chip; whole 128 x (bn_large/2) tiles run on MEDIUM_FULL; everything else on
+// the predicated MEDIUM class.  The pipelined kernels address operands with 32-bit byte offsets.
 int pick_tile(int64_t rows, int64_t cols, int64_t red, int bn_large) {
-  if (rows % 256 == 0 && cols % bn_large == 0 && red % 64 == 0 &&
-      (rows / 256) * (cols / bn_large) >= 192) {
-    static const bool v1 = getenv("GMLP_FORCE_V1") != nullptr;
-    return v1 ? gmlp::TILE_LARGE_V1 : gmlp::TILE_LARGE;
-  }
+  const int64_t limit = (int64_t)1 << 31;
+  bool offsets_fit = rows * red * 2 < limit && cols * red * 2 < limit;
+  if (!offsets_fit || red % 64 != 0) return gmlp::TILE_MEDIUM;
+  if (rows % 256 == 0 && cols % bn_large == 0 && (rows / 256) * (cols / bn_large) >= 192)
+    return gmlp::TILE_LARGE;
+  if (rows % 128 == 0 && cols % (bn_large / 2) == 0) return gmlp::TILE_MEDIUM_FULL;
   return gmlp::TILE_MEDIUM;
 }
 

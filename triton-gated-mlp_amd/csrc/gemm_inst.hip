@@ -1,5 +1,5 @@
 // One translation unit per (dtype, GEMM kind): compiled with -DGMLP_DT=<0|1> -DGMLP_KIND=<0..4>
-// so the kernels build in parallel.  Each unit instantiates the LARGE and MEDIUM tile classes.
+// so the kernels build in parallel.  Each unit instantiates every tile class.
 #include "gemm_v2.hpp"
 #include "launch.hpp"
 
@@ -19,8 +19,8 @@ typedef bf16 DT;
 #define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
   if (tile_class == TILE_LARGE)                                                                  \
     return launch_gemm_v2<DT, 256, BN_L, GMLP_V2_BK, GMLP_V2_NS, 2, 2, AKS, BKS, NB, EPI<DT>>(ga, ea, s); \
-  if (tile_class == TILE_LARGE_V1)                                                               \
-    return launch_gemm<DT, 256, BN_L, 64, 2, 2, AKS, BKS, NB, false, EPI<DT>>(ga, ea, s);         \
+  if (tile_class == TILE_MEDIUM_FULL)                                                            \
+    return launch_gemm_v2<DT, 128, BN_M, GMLP_V2_BK, GMLP_V2_NS, 2, 2, AKS, BKS, NB, EPI<DT>>(ga, ea, s); \
   return launch_gemm<DT, 128, BN_M, 64, 2, 2, AKS, BKS, NB, true, EPI<DT>>(ga, ea, s);
 
 #if GMLP_KIND == 0

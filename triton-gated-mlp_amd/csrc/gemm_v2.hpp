@@ -47,7 +47,7 @@ struct TileV2 {
   // lane fetches with the wavefront's i-th load instruction.  Constant for the whole kernel.
   static __device__ __forceinline__ uint32_t lane_offset(int i, int ld, int wave, int lane) {
     int I = wave * PER_WAVE + i;
-    if (!KS) {
+    if constexpr (!KS) {
       int row = I * RPI_KC + lane / CPR_KC, pos = lane % CPR_KC;
       int c = pos ^ swz_kc(row);
       return (uint32_t)(row * ld + c * 8) * 2u;
@@ -63,7 +63,7 @@ struct TileV2 {
 
   // MFMA fragment (8 reduction elements per lane) for rows row0..row0+31, reduction step ks.
   static __device__ __forceinline__ vec8 frag(const char* lds_tile, int row0, int ks, int lane) {
-    if (!KS) {
+    if constexpr (!KS) {
       int row = row0 + (lane & 31);
       int c = ks * 2 + (lane >> 5);
       return *(const vec8*)(lds_tile + row * (BK * 2) + ((c ^ swz_kc(row)) << 4));
@@ -203,7 +203,7 @@ __device__ __forceinline__ void gemm_v2_body(const GemmArgs& ga, const typename 
   // So the step is laid out as NMFMA slots of {one MFMA; one operand read for the next step, or a
   // share of the global->LDS loads of a tile}, and the scheduler is told to keep the slots.
   constexpr int NMFMA = NB * TM * TN;
-  static_assert(NFRAG < NMFMA, "operand reads must fit in the MFMA slots");
+  static_assert(NFRAG <= NMFMA, "operand reads must fit in the MFMA slots");
   // The refill of a ring slot starts in the step that retires it and is paced at one load per
   // LOAD_STRIDE slots (the vector-memory front end takes a 1 KiB wavefront load every ~16 cycles
   // for the whole CU; issuing faster blocks the wavefront, and the MFMAs queued behind it).

@@ -5,9 +5,12 @@
 
 namespace gmlp {
 
-// Tile classes.  LARGE: 256x256x64 output tiles, 4 wavefronts of 128x128 (full tiles only).
-// MEDIUM: 128x128x64, 4 wavefronts of 64x64, with edge predication (any M, N%8, K%8).
-enum TileClass { TILE_LARGE = 0, TILE_MEDIUM = 1, TILE_LARGE_V1 = 2 };
+// Tile classes (all four wavefronts per workgroup, 64-wide reduction tiles).
+//   LARGE        256x256 output tiles, wavefronts of 128x128, pipelined kernel, whole tiles only
+//   MEDIUM_FULL  128x128 output tiles, wavefronts of 64x64, pipelined kernel, whole tiles only;
+//                two workgroups per CU, for problems with too few 256x256 tiles to fill the chip
+//   MEDIUM       128x128, predicated register-staged kernel: any M, N % 8, K % 8
+enum TileClass { TILE_LARGE = 0, TILE_MEDIUM = 1, TILE_MEDIUM_FULL = 2 };
 
 // kinds of GEMM the gated MLP needs; each is instantiated per dtype and tile class.
 template <typename T>
