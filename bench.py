@@ -111,6 +111,39 @@ def _decode_line(dev, reps=20):
             "gbps": round(nbytes / avg / 1e6, 1), "frac_hbm_peak": round(nbytes / avg / 1e6 / PEAK_HBM_GBPS, 4)}
 
 
+def _other_configs(dev):
+    """The remaining baseline configurations, timed with events (median of 10 after 3 warm-ups)."""
+    from triton_gated_mlp import FusedGatedMLP
+
+    out = {}
+    for name, (m, k, n, dt, bias, p, bwd) in {
+        "cfg2_fp16_fwd_M4096_K4096_N11008": (4096, 4096, 11008, torch.float16, False, 0.0, False),
+        "cfg4_bf16_fwdbwd_bias_dropout_M2048_K2048_N5632": (2048, 2048, 5632, torch.bfloat16, True, 0.1, True),
+    }.items():
+        mlp = FusedGatedMLP(hidden_size=k, intermediate_size=n, bias=bias, dropout_p=p).to(dev).to(dt)
+        mlp.train(bwd)
+        mlp.dropout_seed = 1234
+        x = torch.randn(m, k, device=dev, dtype=dt, requires_grad=bwd)
+        dy = torch.randn(m, k, device=dev, dtype=dt)
+        params = list(mlp.parameters())
+
+        def step():
+            if bwd:
+                x.grad = None
+                for q in params:
+                    q.grad = None
+                mlp(x).backward(dy)
+            else:
+                with torch.no_grad():
+                    mlp(x)
+
+        avg, med = _event_time_ms(step, 10, warmup=3)
+        flop = (18.0 if bwd else 6.0) * m * n * k
+        out[name] = {"ms": round(med, 4), "tflops": round(flop / med / 1e9, 1),
+                     "frac_mfma_peak": round(flop / med / 1e9 / PEAK_MFMA_F16_TFLOPS, 4)}
+    return out
+
+
 def _cpu_baseline():
     """CPU oracle (fp32 restatement of the eager module, closed-form backward) on a bounded sample:
     the first 1024 of the 8192 token rows, same K and N, forward+backward."""
@@ -225,6 +258,7 @@ def main():
     if not args.no_extras:
         line["kernels"] = _kernel_breakdown(mlp, x, dY, 10)
         line["decode"] = _decode_line(dev)
+        line["other_configs"] = _other_configs(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline()
     print(json.dumps(line), flush=True)

@@ -252,6 +252,25 @@ def test_full_size_properties_cfg3_linearity_and_zero():
     assert not z.hidden.any()
 
 
+def test_memory_lean_backward_is_bit_identical():
+    """recompute_activations=True (keep x only, as the reference does) gives the same gradients."""
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    torch.manual_seed(4)
+    mlp = FusedGatedMLP(512, 1024, bias=True, dropout_p=0.2).to(dev).to(torch.bfloat16).train()
+    x = torch.randn(384, 512, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(384, 512, device=dev, dtype=torch.bfloat16)
+    grads = []
+    for lean in (False, True):
+        mlp.recompute_activations = lean
+        mlp.dropout_seed, mlp._dropout_calls = 77, 0
+        y = mlp(x)
+        grads.append((y, *torch.autograd.grad(y, [x, *mlp.parameters()], grad_outputs=dy)))
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
 def test_grouped_weight_gradients_equal_single_launches():
     """gmlp_dw_bwd_grouped (one grid) is bit-identical to three gmlp_dw_bwd launches."""
     from triton_gated_mlp.ops import bwd as ops_bwd

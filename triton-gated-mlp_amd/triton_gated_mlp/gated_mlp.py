@@ -128,20 +128,31 @@ class FusedGatedMLPFullFunction(Function):
     """Whole MLP as one autograd node, so dY -> (dG, dU) is a single GEMM with a fused epilogue."""
 
     @staticmethod
-    def forward(ctx, x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset):
+    def forward(ctx, x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset, recompute=False):
         needs_grad = any(ctx.needs_input_grad[:7])
-        hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=needs_grad)
+        keep = needs_grad and not recompute
+        hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=keep)
         y = _fwd.linear_fwd(hs.hidden, W_down, b_down)
-        if needs_grad:
+        if keep:
             ctx.save_for_backward(x, W_gate, W_up, W_down, hs.gate, hs.up, hs.hidden)
+        elif needs_grad:
+            # memory-lean mode: keep the inputs only (as the reference does, gated_mlp.py:182) and
+            # run the gate/up GEMM again in backward; the dropout mask is a function of the seed
+            ctx.save_for_backward(x, W_gate, W_up, W_down, b_gate, b_up)
+        ctx.recompute = bool(recompute)
         ctx.dropout = (float(dropout_p), int(seed), int(offset))
         ctx.has_bias = (b_gate is not None, b_up is not None, b_down is not None)
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, W_gate, W_up, W_down, gate, up, hidden = ctx.saved_tensors
         p, seed, offset = ctx.dropout
+        if ctx.recompute:
+            x, W_gate, W_up, W_down, b_gate, b_up = ctx.saved_tensors
+            hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, p, seed, offset, save_activations=True)
+            gate, up, hidden = hs.gate, hs.up, hs.hidden
+        else:
+            x, W_gate, W_up, W_down, gate, up, hidden = ctx.saved_tensors
         need = ctx.needs_input_grad
         dy = dy.contiguous()
         dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
@@ -165,7 +176,7 @@ class FusedGatedMLPFullFunction(Function):
             dW_gate, dW_up, dW_down = grads.get("gate"), grads.get("up"), grads.get("down")
         if ctx.has_bias[2] and need[6]:
             db_down = _bwd.colsum(dy)
-        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None
+        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None, None
 
 
 class FusedGatedMLP(_GatedMLPBase):
@@ -175,6 +186,9 @@ class FusedGatedMLP(_GatedMLPBase):
     set `dropout_seed` (int) for a fixed mask stream, otherwise each forward draws a seed from
     torch's default CPU generator (so `torch.manual_seed` makes runs repeatable).  The seed and
     offset of the last training forward are kept in `last_dropout_state`.
+
+    `recompute_activations = True` selects the memory-lean backward: only x is kept from the forward
+    pass and G, U, H are recomputed (one more gate/up GEMM) instead of holding 3*M*N elements.
     """
 
     def __init__(self, *args, **kwargs):
@@ -184,6 +198,7 @@ class FusedGatedMLP(_GatedMLPBase):
                 f"FusedGatedMLP implements hidden_act='silu' only, got {self.act_fn!r}; use EagerGatedMLP"
             )
         self.dropout_seed: Optional[int] = None
+        self.recompute_activations = False
         self._dropout_calls = 0
         self.last_dropout_state = (0, 0)
 
@@ -210,6 +225,7 @@ class FusedGatedMLP(_GatedMLPBase):
         else:
             seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
             y = FusedGatedMLPFullFunction.apply(
-                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p, seed, offset
+                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p, seed, offset,
+                self.recompute_activations,
             )
         return y.reshape(*lead, self.hidden_size)
