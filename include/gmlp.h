@@ -10,7 +10,8 @@
  *   - All matrices are dense, row-major, contiguous, on the current HIP device, 16-byte aligned.
  *   - M = tokens (rows of x), K = hidden_size, N = intermediate_size.
  *     W_gate, W_up are [N,K]; W_down is [K,N]  (torch.nn.Linear [out,in] layout).
- *   - dtype: GMLP_F16 or GMLP_BF16 storage; accumulation and epilogue arithmetic are fp32.
+ *   - dtype: GMLP_F16 or GMLP_BF16 storage (the tuned kernels) or GMLP_F32 (compatibility path on
+ *     fp32 MFMA, not tuned; not for gmlp_decode_fwd); accumulation and epilogue arithmetic are fp32.
  *   - Every call only ENQUEUES work on `stream` (a hipStream_t; NULL = default stream) and returns.
  *     The library never allocates, frees or keeps device memory; the caller owns every buffer,
  *     including workspaces (sizes from gmlp_workspace_bytes).
@@ -32,7 +33,7 @@ extern "C" {
 
 #define GMLP_ABI_VERSION 1
 
-enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1 };
+enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
 enum gmlp_status {
   GMLP_OK = 0,

@@ -252,6 +252,84 @@ def test_full_size_properties_cfg3_linearity_and_zero():
     assert not z.hidden.any()
 
 
+# ---- float32: the reference's own four tests run in float32 (tests/test_gated_mlp_fwd.py:23-82,
+# tests/test_gated_mlp_bwd.py:27-129); same shapes, inputs and tolerances here.
+
+
+def test_reference_fp32_module_forward():
+    from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP, copy_weights
+
+    dev = _dev()
+    torch.manual_seed(0)
+    eager = EagerGatedMLP(dropout_p=0.0).to(dev).float()  # defaults: K=256, N=512, bias=True
+    fused = FusedGatedMLP(dropout_p=0.0).to(dev).float()
+    copy_weights(eager, fused)
+    x = torch.rand((128, eager.hidden_size), device=dev, dtype=torch.float32)
+    y_e, y_f = eager(x), fused(x)
+    assert torch.allclose(y_f, y_e, rtol=1e-6, atol=1e-2)  # the reference's effective tolerance
+    assert torch.allclose(y_f, y_e, rtol=1e-4, atol=1e-5)  # what fp32 accumulation actually gives
+    ref = oracle.forward(x.cpu().double(), *[t.detach().cpu().double() for t in (
+        eager.gate_proj.weight, eager.gate_proj.bias, eager.up_proj.weight, eager.up_proj.bias,
+        eager.down_proj.weight, eager.down_proj.bias)])["Y"]
+    assert torch.allclose(y_f.cpu().double(), ref, rtol=1e-4, atol=1e-5)
+
+
+def test_reference_fp32_operator_forward():
+    from triton_gated_mlp import EagerGatedMLP, eager_fwd, mlp_hidden_states_fwd
+
+    dev = _dev()
+    torch.manual_seed(1)
+    m = EagerGatedMLP(dropout_p=0.0, bias=False).to(dev).float()
+    x = torch.rand((128, m.hidden_size), device=dev)
+    ref = eager_fwd(x, m.up_proj.weight, None, m.gate_proj.weight, None)
+    out = mlp_hidden_states_fwd(x, m.up_proj.weight, None, m.gate_proj.weight, None, m.act_fn, m.dropout.p)
+    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_reference_fp32_module_backward_3d_input():
+    from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP, copy_weights
+
+    dev = _dev()
+    torch.manual_seed(2)
+    eager = EagerGatedMLP(dropout_p=0.0, bias=False).to(dev).float()
+    fused = FusedGatedMLP(dropout_p=0.0, bias=False).to(dev).float()
+    copy_weights(eager, fused)
+    x = torch.rand((16, 32, eager.hidden_size), device=dev, requires_grad=True)
+    y_e, y_f = eager(x), fused(x)
+    assert y_f.shape == x.shape
+    assert torch.allclose(y_f, y_e, atol=1e-3)
+    go = torch.rand_like(x)
+    g_e = torch.autograd.grad(y_e, (x, eager.up_proj.weight, eager.gate_proj.weight, eager.down_proj.weight), grad_outputs=go)
+    g_f = torch.autograd.grad(y_f, (x, fused.up_proj.weight, fused.gate_proj.weight, fused.down_proj.weight), grad_outputs=go)
+    for a, b in zip(g_f, g_e):
+        rel = ((a - b).norm() / b.norm()).item()
+        assert rel < 1e-5, rel
+
+
+def test_reference_fp32_operator_backward():
+    from triton_gated_mlp import mlp_hidden_states_bwd
+
+    dev = _dev()
+    torch.manual_seed(3)
+    B, M, N, K = 2, 32, 512, 256
+    kw = dict(device=dev, dtype=torch.float32)
+    x = torch.rand((B * M, K), **kw) / K
+    W_up, W_gp = torch.rand((N, K), **kw) / K, torch.rand((N, K), **kw) / K
+    go = torch.rand((B * M, N), **kw) / K
+    a, b = x @ W_up.T, x @ W_gp.T
+    sig = torch.sigmoid(b)
+    goap = go * a * (sig * (1 + b * (1 - sig)))
+    goc = go * torch.nn.functional.silu(b)
+    dx, dW_up, dW_gp = mlp_hidden_states_bwd(x, W_up, W_gp, go)
+    for got, ref in ((dx, goc @ W_up + goap @ W_gp), (dW_up, goc.T @ x), (dW_gp, goap.T @ x)):
+        rel = ((got - ref).norm() / ref.norm()).item()
+        assert rel < 1e-5, rel  # the reference asks 1e-7 of its own kernels; fp32 MFMA order differs from BLAS
+
+
+def test_fp32_bias_dropout_forward_backward_against_oracle():
+    _run_module_case(Case("fp32_200x136x264", 200, 136, 264, torch.float32, bias=True, p=0.25, backward=True, seed=5))
+
+
 def test_memory_lean_backward_is_bit_identical():
     """recompute_activations=True (keep x only, as the reference does) gives the same gradients."""
     from triton_gated_mlp import FusedGatedMLP

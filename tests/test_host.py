@@ -45,8 +45,9 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     err = lambda: lib.gmlp_last_error().decode()
     # NULL pointer
     assert lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None) == -1 and "NULL" in err()
-    # bad dtype
+    # bad dtype; float32 is not available for the skinny-M kernels
     assert lib.gmlp_linear_fwd(a, a, None, a, 8, 8, 8, 7, None) == -1 and "dtype" in err()
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 256, 2, None) == -2
     # shape: K not a multiple of 8, M < 1
     assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None) == -2 and "multiple of 8" in err()
     assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0.0, 0, 0, None) == -2
@@ -79,8 +80,9 @@ def test_error_codes_map_to_python_exceptions():
         _cabi.check(lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None))
     with pytest.raises(ValueError, match="NULL"):
         _cabi.check(lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None))
-    with pytest.raises(TypeError, match="float16 or bfloat16"):
-        _cabi.dtype_code(torch.float32)
+    with pytest.raises(TypeError, match="float16, bfloat16 or float32"):
+        _cabi.dtype_code(torch.float64)
+    assert [_cabi.dtype_code(t) for t in (torch.float16, torch.bfloat16, torch.float32)] == [0, 1, 2]
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -29,8 +29,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
   if ((p) != nullptr && !aligned16(p))                                              \
   return fail(GMLP_EALIGN, "%s: argument '%s' is not 16-byte aligned", __func__, #p)
 #define GMLP_REQUIRE_DTYPE(d)                                                       \
-  if ((d) != GMLP_F16 && (d) != GMLP_BF16)                                          \
-  return fail(GMLP_EINVAL, "%s: dtype %d is not GMLP_F16/GMLP_BF16", __func__, (int)(d))
+  if ((d) != GMLP_F16 && (d) != GMLP_BF16 && (d) != GMLP_F32)                       \
+  return fail(GMLP_EINVAL, "%s: dtype %d is not GMLP_F16/GMLP_BF16/GMLP_F32", __func__, (int)(d))
 
 const int64_t kMaxDim = (int64_t)1 << 30;
 
@@ -61,6 +61,14 @@ int make_dropout(const char* fn, float p, uint64_t seed, uint64_t offset, gmlp::
   d->off_lo = (uint32_t)offset;
   d->off_hi = (uint32_t)(offset >> 32);
   return 0;
+}
+
+// Calls f(T{}) with T = the storage type named by `dtype` (already validated).
+template <typename F>
+hipError_t by_dtype(int dtype, F&& f) {
+  if (dtype == GMLP_F16) return f(gmlp::f16{});
+  if (dtype == GMLP_BF16) return f(gmlp::bf16{});
+  return f(float{});
 }
 
 int hip_result(const char* fn, hipError_t e) {
@@ -117,16 +125,12 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(M, N, K, 128);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    EpiGateUp<f16>::Args ea = {(f16*)h, (f16*)g_save, (f16*)u_save, mask_out, (const f16*)b_gate,
-                               (const f16*)b_up, (int)N, d};
-    e = launch_gateup<f16>(tc, ga, ea, s);
-  } else {
-    EpiGateUp<bf16>::Args ea = {(bf16*)h, (bf16*)g_save, (bf16*)u_save, mask_out,
-                                (const bf16*)b_gate, (const bf16*)b_up, (int)N, d};
-    e = launch_gateup<bf16>(tc, ga, ea, s);
-  }
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    typename EpiGateUp<T>::Args ea = {(T*)h, (T*)g_save, (T*)u_save, mask_out, (const T*)b_gate,
+                                      (const T*)b_up, (int)N, d};
+    return launch_gateup<T>(tc, ga, ea, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -147,14 +151,11 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(M, C, R, 256);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    EpiStore<f16>::Args ea = {(f16*)out, (const f16*)bias, (int)C};
-    e = launch_linear<f16>(tc, ga, ea, s);
-  } else {
-    EpiStore<bf16>::Args ea = {(bf16*)out, (const bf16*)bias, (int)C};
-    e = launch_linear<bf16>(tc, ga, ea, s);
-  }
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    typename EpiStore<T>::Args ea = {(T*)out, (const T*)bias, (int)C};
+    return launch_linear<T>(tc, ga, ea, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -180,14 +181,11 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(M, N, K, 256);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    EpiDh<f16>::Args ea = {(const f16*)g, (const f16*)u, (f16*)dg, (f16*)du, (int)N, d};
-    e = launch_dh<f16>(tc, ga, ea, s);
-  } else {
-    EpiDh<bf16>::Args ea = {(const bf16*)g, (const bf16*)u, (bf16*)dg, (bf16*)du, (int)N, d};
-    e = launch_dh<bf16>(tc, ga, ea, s);
-  }
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    typename EpiDh<T>::Args ea = {(const T*)g, (const T*)u, (T*)dg, (T*)du, (int)N, d};
+    return launch_dh<T>(tc, ga, ea, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -205,11 +203,10 @@ int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void
   GMLP_REQUIRE_ALIGNED(dh); GMLP_REQUIRE_ALIGNED(g); GMLP_REQUIRE_ALIGNED(u);
   GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = dtype == GMLP_F16
-                     ? launch_gating_bwd<f16>((const f16*)dh, (const f16*)g, (const f16*)u, (f16*)dg,
-                                              (f16*)du, M, N, d, s)
-                     : launch_gating_bwd<bf16>((const bf16*)dh, (const bf16*)g, (const bf16*)u,
-                                               (bf16*)dg, (bf16*)du, M, N, d, s);
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    return launch_gating_bwd<T>((const T*)dh, (const T*)g, (const T*)u, (T*)dg, (T*)du, M, N, d, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -232,14 +229,11 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   ga.nseg = 2; ga.group_m = 8;
   int tc = pick_tile(M, K, N, 256);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    EpiStore<f16>::Args ea = {(f16*)dx, nullptr, (int)K};
-    e = launch_dx<f16>(tc, ga, ea, s);
-  } else {
-    EpiStore<bf16>::Args ea = {(bf16*)dx, nullptr, (int)K};
-    e = launch_dx<bf16>(tc, ga, ea, s);
-  }
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};
+    return launch_dx<T>(tc, ga, ea, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -260,14 +254,11 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(R, C, Mred, 256);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    EpiStore<f16>::Args ea = {(f16*)dw, nullptr, (int)C};
-    e = launch_dw<f16>(tc, ga, ea, s);
-  } else {
-    EpiStore<bf16>::Args ea = {(bf16*)dw, nullptr, (int)C};
-    e = launch_dw<bf16>(tc, ga, ea, s);
-  }
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    typename EpiStore<T>::Args ea = {(T*)dw, nullptr, (int)C};
+    return launch_dw<T>(tc, ga, ea, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -286,7 +277,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     if (int rc = check_mult8(__func__, "R", R[i])) return rc;
     if (int rc = check_mult8(__func__, "C", C[i])) return rc;
     GMLP_REQUIRE_ALIGNED(lhs[i]); GMLP_REQUIRE_ALIGNED(rhs[i]); GMLP_REQUIRE_ALIGNED(dw[i]);
-    large = large && pick_tile(R[i], C[i], Mred, 256) == TILE_LARGE;
+    large = large && dtype != GMLP_F32 && pick_tile(R[i], C[i], Mred, 256) == TILE_LARGE;
   }
   if (!large) {
     for (int i = 0; i < count; ++i)
@@ -330,9 +321,10 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
   if (int rc = check_mult8(__func__, "C", C)) return rc;
   GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(out); GMLP_REQUIRE_ALIGNED(workspace);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = dtype == GMLP_F16
-                     ? launch_colsum<f16>((const f16*)a, (f16*)out, (float*)workspace, M, C, s)
-                     : launch_colsum<bf16>((const bf16*)a, (bf16*)out, (float*)workspace, M, C, s);
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    return launch_colsum<T>((const T*)a, (T*)out, (float*)workspace, M, C, s);
+  });
   return hip_result(__func__, e);
 }
 
@@ -346,6 +338,7 @@ int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const v
   GMLP_REQUIRE_PTR(h_scratch); GMLP_REQUIRE_PTR(y);
   GMLP_REQUIRE_DTYPE(dtype);
   if (int rc = check_dims(__func__, M, K, N)) return rc;
+  if (dtype == GMLP_F32) return fail(GMLP_ESHAPE, "%s: float32 is not supported by the skinny-M kernels", __func__);
   if (M > 16) return fail(GMLP_ESHAPE, "%s: M = %lld exceeds the skinny-M limit of 16", __func__, (long long)M);
   if (K % 32 != 0) return fail(GMLP_ESHAPE, "%s: K = %lld must be a multiple of 32", __func__, (long long)K);
   if (N % 256 != 0) return fail(GMLP_ESHAPE, "%s: N = %lld must be a multiple of 256", __func__, (long long)N);

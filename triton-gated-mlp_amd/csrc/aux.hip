@@ -32,6 +32,9 @@ template hipError_t launch_gating_bwd<f16>(const f16*, const f16*, const f16*, f
                                            int64_t, const DropoutParams&, hipStream_t);
 template hipError_t launch_gating_bwd<bf16>(const bf16*, const bf16*, const bf16*, bf16*, bf16*,
                                             int64_t, int64_t, const DropoutParams&, hipStream_t);
+template hipError_t launch_gating_bwd<float>(const float*, const float*, const float*, float*,
+                                             float*, int64_t, int64_t, const DropoutParams&,
+                                             hipStream_t);
 
 // Column sums in two fixed-order stages: COLSUM_SPLITS row ranges -> fp32 partials -> total.
 constexpr int COLSUM_SPLITS = 64;
@@ -77,6 +80,7 @@ hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hi
 }
 template hipError_t launch_colsum<f16>(const f16*, f16*, float*, int64_t, int64_t, hipStream_t);
 template hipError_t launch_colsum<bf16>(const bf16*, bf16*, float*, int64_t, int64_t, hipStream_t);
+template hipError_t launch_colsum<float>(const float*, float*, float*, int64_t, int64_t, hipStream_t);
 
 __global__ void __launch_bounds__(256)
     dropout_mask_kernel(uint8_t* __restrict__ mask, size_t n4, DropoutParams d) {

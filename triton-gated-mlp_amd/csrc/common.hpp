@@ -45,6 +45,14 @@ struct Traits<bf16> {
   static __device__ __forceinline__ bf16 from_f32(float v) { return (bf16)v; }
 };
 
+template <>
+struct Traits<float> {
+  typedef float vec8 __attribute__((ext_vector_type(8)));
+  typedef float vec4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ float to_f32(float v) { return v; }
+  static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+
 // sigma(x) = 1/(1+e^-x), silu(x) = x*sigma(x), silu'(x) = sigma*(1 + x*(1-sigma)); all fp32.
 // Same forms as the reference's _compute_sigma/_silu_fwd/_silu_bwd (src/triton_gated_mlp/ops/act.py:28-45).
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }

@@ -14,7 +14,7 @@ from typing import Optional
 import torch
 from torch import Tensor
 
-GMLP_F16, GMLP_BF16 = 0, 1
+GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM = 0, 1
 ABI_VERSION = 1
 
@@ -88,10 +88,9 @@ def dtype_code(dtype: torch.dtype) -> int:
         return GMLP_F16
     if dtype == torch.bfloat16:
         return GMLP_BF16
-    raise TypeError(
-        f"fused gated-MLP kernels take float16 or bfloat16 tensors, got {dtype}; "
-        "cast the module and its input (e.g. .to(torch.float16))"
-    )
+    if dtype == torch.float32:
+        return GMLP_F32
+    raise TypeError(f"fused gated-MLP kernels take float16, bfloat16 or float32 tensors, got {dtype}")
 
 
 def require_gpu(*tensors: Optional[Tensor]) -> torch.device:

@@ -180,7 +180,8 @@ class FusedGatedMLPFullFunction(Function):
 
 
 class FusedGatedMLP(_GatedMLPBase):
-    """Drop-in gated MLP running on hand-written gfx950 kernels (float16 / bfloat16).
+    """Drop-in gated MLP running on hand-written gfx950 kernels (float16 / bfloat16 tuned; float32
+    on a compatibility path).
 
     Dropout is active in training mode only.  The keep mask comes from a counter-based generator:
     set `dropout_seed` (int) for a fixed mask stream, otherwise each forward draws a seed from
@@ -220,7 +221,7 @@ class FusedGatedMLP(_GatedMLPBase):
         inference = not torch.is_grad_enabled() or not (
             x2.requires_grad or any(q.requires_grad for q in self.parameters())
         )
-        if inference and p == 0.0 and _fwd.decode_supported(M, K, self.intermediate_size):
+        if inference and p == 0.0 and _fwd.decode_supported(M, K, self.intermediate_size, x2.dtype):
             y = _fwd.decode_fwd(x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias)
         else:
             seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)

@@ -122,8 +122,8 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
 DECODE_MAX_M = 16
 
 
-def decode_supported(M: int, K: int, N: int) -> bool:
-    return 1 <= M <= DECODE_MAX_M and K % 32 == 0 and N % 256 == 0
+def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16) -> bool:
+    return dtype in (torch.float16, torch.bfloat16) and 1 <= M <= DECODE_MAX_M and K % 32 == 0 and N % 256 == 0
 
 
 def decode_fwd(
