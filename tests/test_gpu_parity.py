@@ -330,6 +330,67 @@ def test_fp32_bias_dropout_forward_backward_against_oracle():
     _run_module_case(Case("fp32_200x136x264", 200, 136, 264, torch.float32, bias=True, p=0.25, backward=True, seed=5))
 
 
+def test_empty_and_degenerate_inputs():
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    torch.manual_seed(6)
+    mlp = FusedGatedMLP(256, 512, bias=True).to(dev).half()
+    # no tokens
+    x0 = torch.zeros(0, 256, device=dev, dtype=torch.float16, requires_grad=True)
+    y0 = mlp(x0)
+    assert y0.shape == (0, 256)
+    g = torch.autograd.grad(y0, [x0, mlp.gate_proj.weight, mlp.down_proj.bias], grad_outputs=torch.zeros_like(y0))
+    assert g[0].shape == (0, 256) and not g[1].any() and not g[2].any()
+    assert mlp(torch.zeros(4, 0, 256, device=dev, dtype=torch.float16)).shape == (4, 0, 256)
+    # leading dimensions of one and a single token, with gradients
+    x1 = torch.randn(1, 1, 256, device=dev, dtype=torch.float16, requires_grad=True)
+    y1 = mlp(x1)
+    (gx,) = torch.autograd.grad(y1, [x1], grad_outputs=torch.ones_like(y1))
+    f = lambda t: t.detach().float().cpu()
+    ref = oracle.backward(f(x1).view(1, 256), f(mlp.gate_proj.weight), f(mlp.gate_proj.bias), f(mlp.up_proj.weight),
+                          f(mlp.up_proj.bias), f(mlp.down_proj.weight), f(mlp.down_proj.bias), torch.ones(1, 256))
+    _close("Y single token", y1.view(1, 256), ref["Y"])
+    _close("dX single token", gx.view(1, 256), ref["dX"])
+
+
+def test_non_contiguous_inputs_and_partial_gradients():
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    torch.manual_seed(7)
+    mlp = FusedGatedMLP(256, 768, bias=False).to(dev).to(torch.bfloat16)
+    base = torch.randn(96, 512, device=dev, dtype=torch.bfloat16)
+    x_nc = base[:, ::2]  # stride 2 along the feature dimension
+    assert not x_nc.is_contiguous()
+    y_nc = mlp(x_nc)
+    assert torch.equal(y_nc, mlp(x_nc.contiguous()))
+    # only the input needs a gradient (weights frozen): no weight-gradient launches, same dX
+    x = x_nc.contiguous().requires_grad_(True)
+    y = mlp(x)
+    dy = torch.randn_like(y)
+    (dx_full,) = torch.autograd.grad(y, [x], grad_outputs=dy, retain_graph=True)
+    for q in mlp.parameters():
+        q.requires_grad_(False)
+    (dx_frozen,) = torch.autograd.grad(mlp(x), [x], grad_outputs=dy)
+    assert torch.equal(dx_full, dx_frozen)
+    # only the weights need a gradient
+    for q in mlp.parameters():
+        q.requires_grad_(True)
+    xw = x.detach()
+    gw = torch.autograd.grad(mlp(xw), list(mlp.parameters()), grad_outputs=dy)
+    f = lambda t: t.detach().float().cpu()
+    ref = oracle.backward(f(xw), f(mlp.gate_proj.weight), None, f(mlp.up_proj.weight), None, f(mlp.down_proj.weight),
+                          None, f(dy))
+    for n, got in zip(("dW_gate", "dW_up", "dW_down"), gw):
+        _close(n, got, ref[n], atol=ATOL * 4)
+
+
+def test_many_tokens_tall_shape():
+    """M much larger than K and N (65536 tokens): 32-bit index paths and the tile scheduler."""
+    _run_module_case(Case("tall_65536x256x512", 65536, 256, 512, torch.float16, bias=False, backward=True, seed=8))
+
+
 def test_memory_lean_backward_is_bit_identical():
     """recompute_activations=True (keep x only, as the reference does) gives the same gradients."""
     from triton_gated_mlp import FusedGatedMLP

@@ -219,13 +219,7 @@ template <typename T, bool GATED>
 static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
   constexpr int LDS = DS_WAVES * DS_RD * 2 * DS_REGION + 2 * (DS_WAVES - 1) * 2 * 256 * 4;
   auto kern = decode_stream_kernel<T, GATED>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS)) return e;
   int nblocks = a.R / (GATED ? 16 : 32);
   int grid = nblocks < num_cu ? nblocks : num_cu;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);
@@ -241,15 +235,10 @@ template <typename T>
 hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
                                 const T* bu, const T* bd, T* h, T* y, int M, int K, int N,
                                 hipStream_t s) {
-  static int num_cu = 0;
-  if (num_cu == 0) {
-    int dev = 0, n = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    num_cu = n > 0 ? n : 256;
-  }
+  int dev = 0, num_cu = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  if (hipError_t e = hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+  if (num_cu <= 0) num_cu = 256;
   StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N};
   hipError_t e = launch_stream<T, true>(a1, num_cu, s);
   if (e != hipSuccess) return e;

@@ -86,6 +86,12 @@ struct TileV2 {
   }
 };
 
+// Raises the dynamic-LDS limit of `kernel` on the current device (needed above 64 KiB).  Called on
+// every launch: the attribute is per device, and the call only touches host-side state.
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
+  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_KS, bool B_KS,
           int NB>
 struct ConfigV2 {
@@ -346,13 +352,7 @@ template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_K
 hipError_t launch_gemm_group_v2(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
   typedef ConfigV2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_group_kernel_v2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
   int total = 0;
   for (int g = 0; g < grp.count; ++g) {
     grp.first[g] = total;
@@ -368,13 +368,7 @@ template <typename T, int BM, int BN, int BK, int NS, int WGM, int WGN, bool A_K
 hipError_t launch_gemm_v2(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
   typedef ConfigV2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_kernel_v2<T, BM, BN, BK, NS, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
   dim3 grid((ga.M / BM) * (ga.N / BN)), block(Cfg::NW * 64);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
   return hipGetLastError();
