@@ -230,7 +230,7 @@ def main():
     xd = x.detach()
     avg, med = _event_time_ms(lambda: F.gateup_fwd(xd, Wg, None, Wu, None, save_activations=True), max(args.steps, 10))
     dom_flop = 4.0 * M * N * K
-    roofline = {"kernel": "gemm_kernel<f16,256,128,64,...,EpiGateUp> (gate/up forward GEMM + SiLU-gating epilogue)",
+    roofline = {"kernel": "gemm_kernel_pipelined<f16,256,128,16,...,EpiGateUp> (gate/up forward GEMM + SiLU-gating epilogue)",
                 "bound": "mfma", "achieved": round(dom_flop / avg / 1e9, 1), "peak": PEAK_MFMA_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_flop / avg / 1e9 / PEAK_MFMA_F16_TFLOPS, 4),
                 "avg_launch_ms": round(avg, 4), "flop_per_launch": dom_flop, "traffic": GATEUP_TRAFFIC_BYTES,

@@ -17,7 +17,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Per-dtype traits.  An operand fragment of v_mfma_f32_32x32x16_{f16,bf16} is 8 consecutive
+// Per-dtype traits.  mfma = v_mfma_f32_32x32x16, mfma16 = v_mfma_f32_16x16x32 (4 accumulator floats
+// per lane: column l % 16, rows 4*(l/16) .. +3).  An operand fragment of v_mfma_f32_32x32x16_{f16,bf16} is 8 consecutive
 // reduction elements per lane: lane l carries row (l % 32), reduction slots 8*(l / 32) .. +7.
 // The 16 accumulator floats of lane l sit at column (l % 32), rows 8*(i/4) + 4*(l/32) + (i%4).
 template <typename T>
@@ -30,6 +31,9 @@ struct Traits<f16> {
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ float to_f32(f16 v) { return (float)v; }
   static __device__ __forceinline__ f16 from_f32(float v) { return (f16)v; }
 };
@@ -40,6 +44,9 @@ struct Traits<bf16> {
   typedef bf16x4 vec4;
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ float to_f32(bf16 v) { return (float)v; }
   static __device__ __forceinline__ bf16 from_f32(float v) { return (bf16)v; }

@@ -285,6 +285,17 @@ struct EpiStore {
     if (a.bias) add_w<T, W>(a.bias + n, v);
     store_w<T, W>(a.out + (size_t)m * a.ldc + n, v);
   }
+  // Nothing worth fetching ahead of time (see EpiDh).
+  static constexpr int PREFETCH_DEPTH = 0;
+  template <int W>
+  struct Prefetch {};
+  template <int W>
+  static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float* w,
+                                               const Prefetch<W>&) {
+    apply<W>(a, m, n, v, w);
+  }
 };
 
 // G = acc0 + b_gate, U = acc1 + b_up, H = dropout(silu(G) * U)
@@ -330,15 +341,24 @@ struct EpiGateUp {
     if (a.g_save) store_w<T, W>(a.g_save + e, g);
     if (a.u_save) store_w<T, W>(a.u_save + e, u);
   }
+  static constexpr int PREFETCH_DEPTH = 0;
+  template <int W>
+  struct Prefetch {};
+  template <int W>
+  static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* g, float* u,
+                                               const Prefetch<W>&) {
+    apply<W>(a, m, n, g, u);
+  }
 };
 
 // Gating backward on W consecutive elements: dA = dH*keep/(1-p); dU = dA*silu(G); dG = dA*U*silu'(G)
 template <typename T, int W>
-__device__ __forceinline__ void gating_bwd_w(const DropoutParams& drop, size_t e, float* dh,
-                                             const T* g, const T* u, T* dg, T* du) {
-  float gv[W], uv[W], dgv[W], duv[W];
-  load_w<T, W>(g + e, gv);
-  load_w<T, W>(u + e, uv);
+__device__ __forceinline__ void gating_bwd_core(const DropoutParams& drop, size_t e, float* dh,
+                                                typename PackW<T, W>::type gp,
+                                                typename PackW<T, W>::type up, T* dg, T* du) {
+  float dgv[W], duv[W];
   if (drop.enabled) {
     bool keep[W];
     keep_w<W>(drop, e, keep);
@@ -347,12 +367,19 @@ __device__ __forceinline__ void gating_bwd_w(const DropoutParams& drop, size_t e
   }
 #pragma unroll
   for (int r = 0; r < W; ++r) {
-    float s = sigmoid_f32(gv[r]);
-    duv[r] = dh[r] * (gv[r] * s);
-    dgv[r] = dh[r] * uv[r] * (s * (1.0f + gv[r] * (1.0f - s)));
+    float gv = Traits<T>::to_f32(gp[r]), uv = Traits<T>::to_f32(up[r]);
+    float s = sigmoid_f32(gv);
+    duv[r] = dh[r] * (gv * s);
+    dgv[r] = dh[r] * uv * (s * (1.0f + gv * (1.0f - s)));
   }
   store_w<T, W>(dg + e, dgv);
   store_w<T, W>(du + e, duv);
+}
+template <typename T, int W>
+__device__ __forceinline__ void gating_bwd_w(const DropoutParams& drop, size_t e, float* dh,
+                                             const T* g, const T* u, T* dg, T* du) {
+  typedef typename PackW<T, W>::type pack;
+  gating_bwd_core<T, W>(drop, e, dh, *(const pack*)(g + e), *(const pack*)(u + e), dg, du);
 }
 
 template <typename T>
@@ -368,6 +395,25 @@ struct EpiDh {
   template <int W>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*) {
     gating_bwd_w<T, W>(a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
+  }
+  // G and U come from HBM and every workgroup of a round reaches its epilogue at about the same
+  // time; a kernel that can, fetches them this many W-wide items ahead of their use.
+  static constexpr int PREFETCH_DEPTH = 8;
+  template <int W>
+  struct Prefetch {
+    typename PackW<T, W>::type g, u;
+  };
+  template <int W>
+  static __device__ __forceinline__ void prefetch(const Args& a, int m, int n, Prefetch<W>& p) {
+    typedef typename PackW<T, W>::type pack;
+    size_t e = (size_t)m * a.ldc + n;
+    p.g = *(const pack*)(a.g + e);
+    p.u = *(const pack*)(a.u + e);
+  }
+  template <int W>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*,
+                                               const Prefetch<W>& p) {
+    gating_bwd_core<T, W>(a.drop, (size_t)m * a.ldc + n, dh, p.g, p.u, a.dg, a.du);
   }
 };
 

@@ -1,12 +1,7 @@
 // One translation unit per (dtype, GEMM kind): compiled with -DGMLP_DT=<0|1> -DGMLP_KIND=<0..4>
 // so the kernels build in parallel.  Each unit instantiates every tile class.
-#include "gemm_v2.hpp"
+#include "gemm_pipelined.hpp"
 #include "launch.hpp"
-
-#ifndef GMLP_V2_BK
-#define GMLP_V2_BK 64  // reduction elements per LDS ring slot
-#define GMLP_V2_NS 2   // ring depth
-#endif
 
 namespace gmlp {
 
@@ -16,11 +11,19 @@ typedef f16 DT;
 typedef bf16 DT;
 #endif
 
+#ifndef GMLP_MI
+#define GMLP_MI 16  // MFMA shape: 16 = v_mfma_f32_16x16x32, 32 = v_mfma_f32_32x32x16
+#endif
+#define GMLP_LARGE(AKS, BKS, NB, EPI, BN_L) \
+  launch_gemm_pipelined<DT, 256, BN_L, GMLP_MI, 2, 2, AKS, BKS, NB, EPI<DT>>
+#define GMLP_MEDIUM(AKS, BKS, NB, EPI, BN_M) \
+  launch_gemm_pipelined<DT, 128, BN_M, GMLP_MI, 2, 2, AKS, BKS, NB, EPI<DT>>
+#define GMLP_LARGE_GROUP \
+  launch_gemm_group_pipelined<DT, 256, 256, GMLP_MI, 2, 2, true, true, 1, EpiStore<DT>>
+
 #define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
-  if (tile_class == TILE_LARGE)                                                                  \
-    return launch_gemm_v2<DT, 256, BN_L, GMLP_V2_BK, GMLP_V2_NS, 2, 2, AKS, BKS, NB, EPI<DT>>(ga, ea, s); \
-  if (tile_class == TILE_MEDIUM_FULL)                                                            \
-    return launch_gemm_v2<DT, 128, BN_M, GMLP_V2_BK, GMLP_V2_NS, 2, 2, AKS, BKS, NB, EPI<DT>>(ga, ea, s); \
+  if (tile_class == TILE_LARGE) return GMLP_LARGE(AKS, BKS, NB, EPI, BN_L)(ga, ea, s);           \
+  if (tile_class == TILE_MEDIUM_FULL) return GMLP_MEDIUM(AKS, BKS, NB, EPI, BN_M)(ga, ea, s);    \
   return launch_gemm<DT, 128, BN_M, 64, 2, 2, AKS, BKS, NB, true, EPI<DT>>(ga, ea, s);
 
 #if GMLP_KIND == 0
@@ -55,7 +58,7 @@ hipError_t launch_dw<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>:
 }
 template <>
 hipError_t launch_dw_group<DT>(GemmGroup<EpiStore<DT>::Args>& grp, hipStream_t s) {
-  return launch_gemm_group_v2<DT, 256, 256, GMLP_V2_BK, GMLP_V2_NS, 2, 2, true, true, 1, EpiStore<DT>>(grp, s);
+  return GMLP_LARGE_GROUP(grp, s);
 }
 #endif
 

@@ -1,0 +1,399 @@
+// Pipelined full-tile MFMA GEMM for gfx950.
+//
+// Same contract as gemm_kernel (gemm.hpp): C[M,N] = sum_s sum_k A_s[m,k] * B_s[n,k], operands
+// reduction-contiguous (KC) or reduction-strided (KS), NB accumulator sets, fused epilogue; but
+// restricted to whole BM x BN tiles and K % 64 == 0.  Reduction tiles of 64 elements travel
+// global -> LDS without passing through registers (gemm_tiles.hpp) into a two-slot ring; the
+// epilogue transposes accumulators through LDS so that every global access is a 16-byte,
+// row-contiguous one.
+//
+// Per 512/MI-wide reduction step a wavefront issues G groups of TM MFMAs: group g multiplies one
+// B fragment (accumulator set b, column block j; G = NB * TN) with the step's TM A fragments.
+// Operands roll through registers instead of being double-buffered a whole step at a time:
+//   * A fragments: two banks of TM; during step s, group g fetches A fragment g of step s+1;
+//   * B fragments: a ring of 4; group g fetches the B fragment of group g+2.
+// That is 2*TM + 4 fragments in flight (72 VGPRs for the 16x16x32 shape instead of 128), which is
+// what lets v_mfma_f32_16x16x32 be used with a 128x128 register tile: it moves a fifth fewer
+// register bytes per FLOP than 32x32x16 (4 accumulator floats per lane and instruction instead of
+// 16), and on MI355X, where these kernels run power-limited, that shows up as clock.
+//
+// A reduction tile's ring slot is retired at ONE barrier, placed in the tile's last step where the
+// rolling fetches stop addressing the tile: before group G-2.  After it, groups G-2 and G-1 fetch
+// the next tile's first B fragments and all of its first A fragments, and the global->LDS refill of
+// the freed slot starts, paced over the following MFMA slots.
+#pragma once
+#include "gemm_tiles.hpp"
+
+namespace gmlp {
+
+#ifndef GMLP_LOAD_CYCLES
+#define GMLP_LOAD_CYCLES 64  // one global->LDS load per this many MFMA cycles
+#endif
+
+template <int MI>
+struct AccType;
+template <>
+struct AccType<32> { typedef f32x16 type; };
+template <>
+struct AccType<16> { typedef f32x4 type; };
+
+template <typename T, int MI>
+__device__ __forceinline__ typename AccType<MI>::type mfma_mi(typename Traits<T>::vec8 a,
+                                                              typename Traits<T>::vec8 b,
+                                                              typename AccType<MI>::type c) {
+  if constexpr (MI == 32) return Traits<T>::mfma(a, b, c);
+  else return Traits<T>::mfma16(a, b, c);
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB>
+struct PipeConfig {
+  static constexpr int BK = 64, NS = 2;
+  static constexpr int NW = WGM * WGN;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  static constexpr int TM = WTM / MI, TN = WTN / MI, G = NB * TN;
+  static constexpr int KF = 512 / MI;            // reduction elements per MFMA
+  static constexpr int KSTEPS = BK / KF;
+  static constexpr int MFMA_CYCLES = MI == 32 ? 32 : 16;
+  typedef LdsTile<T, BM, BK, A_KS, NW> ATile;
+  typedef LdsTile<T, BN, BK, B_KS, NW> BTile;
+  static constexpr int STAGE = ATile::BYTES + NB * BTile::BYTES;
+  static constexpr int LOADS = ATile::PER_WAVE + NB * BTile::PER_WAVE;  // per wave per tile
+  static constexpr int EPI_LD = WTN + 4;                                // fp32 staging row
+  static constexpr int EPI_WAVE_BYTES = NB * MI * EPI_LD * 4;
+  static constexpr int MAIN_BYTES = NS * STAGE;
+  static constexpr int LDS_BYTES = MAIN_BYTES > NW * EPI_WAVE_BYTES ? MAIN_BYTES : NW * EPI_WAVE_BYTES;
+  static_assert(G >= 2 && TM >= 2 && TM % 2 == 0, "rolling scheme needs >= 2 groups and an even TM");
+  static_assert((KSTEPS * G) % 4 == 0, "B ring index must be static");
+  static_assert(TM <= G, "one A fetch per group must cover the next step");
+  static_assert(KSTEPS % 2 == 0, "A banks alternate by step and every tile starts on bank 0");
+  static_assert(NS == 2, "the retiring barrier waits for everything in flight");
+};
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+__device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const typename Epi::Args& ea,
+                                             int pid, int nwg) {
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  typedef typename Cfg::ATile ATile;
+  typedef typename Cfg::BTile BTile;
+  typedef typename Traits<T>::vec8 vec8;
+  typedef typename AccType<MI>::type acc_t;
+  constexpr int BK = Cfg::BK, NS = Cfg::NS;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, G = Cfg::G, WTM = Cfg::WTM, WTN = Cfg::WTN;
+  constexpr int KSTEPS = Cfg::KSTEPS, STAGE = Cfg::STAGE, L = Cfg::LOADS;
+  constexpr int LOAD_SLOTS = GMLP_LOAD_CYCLES / Cfg::MFMA_CYCLES;  // MFMA slots per load
+  constexpr int TILE_SLOTS = KSTEPS * G * TM;                         // MFMA slots per tile
+  constexpr int HEAD_SLOTS = 2 * TM;  // slots between the retiring barrier and the tile's end
+  // Fragment fetches sit in slots 0 and 1 of a group; with four or more slots per load the loads
+  // keep away from them.
+  constexpr int LOAD_PHASE = LOAD_SLOTS >= 4 ? 2 : 0;
+  static_assert(LOAD_SLOTS >= 1 && L * LOAD_SLOTS <= TILE_SLOTS, "a tile's loads must fit a tile");
+
+  extern __shared__ __align__(1024) char smem_raw[];
+  char* smem = smem_raw;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  const int tiles_m = ga.M / BM, tiles_n = ga.N / BN;
+  int tm_i, tn_i;
+  map_tile(pid, nwg, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+
+  acc_t acc[G][TM];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < (int)(sizeof(acc_t) / 4); ++r) acc[g][i][r] = 0.f;
+
+  const int kt_seg = ga.K / BK;
+  const int kt_total = kt_seg * ga.nseg;
+
+  // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
+  // Buffer addressing uses 32-bit byte offsets from each operand's base; the host checks sizes.
+  // Up to four consecutive loads of an operand share one LDS base in M0 and differ by the
+  // instruction's immediate offset q*1024; the immediate also moves the global address, so lane
+  // offsets carry DMA_BIAS - q*1024 and the buffer descriptors start DMA_BIAS below the operand.
+  constexpr int DMA_BIAS = 3072;
+  uint32_t aoff[ATile::PER_WAVE], boff[BTile::PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < ATile::PER_WAVE; ++i)
+    aoff[i] = ATile::lane_offset(i, ga.lda, wave, lane) + DMA_BIAS - (i & 3) * 1024;
+#pragma unroll
+  for (int i = 0; i < BTile::PER_WAVE; ++i)
+    boff[i] = BTile::lane_offset(i, ga.ldb, wave, lane) + DMA_BIAS - (i & 3) * 1024;
+  const uint32_t a_step = A_KS ? (uint32_t)BK * ga.lda * 2 : (uint32_t)BK * 2;
+  const uint32_t b_step = B_KS ? (uint32_t)BK * ga.ldb * 2 : (uint32_t)BK * 2;
+  const uint32_t a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
+  const uint32_t b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem;
+  const buffer_rsrc ra[2] = {make_rsrc((const char*)ga.A[0] - DMA_BIAS),
+                             make_rsrc((const char*)ga.A[1] - DMA_BIAS)};
+  const buffer_rsrc rb[2] = {make_rsrc((const char*)ga.B[0] - DMA_BIAS),
+                             make_rsrc((const char*)ga.B[1] - DMA_BIAS)};
+
+  // Global->LDS load number x (0 .. L-1) of this wavefront for reduction tile kt_req: operand and
+  // index within the operand's loads.
+  auto load_index = [](int x) __attribute__((always_inline)) {
+    return x < ATile::PER_WAVE ? x : (x - ATile::PER_WAVE) % BTile::PER_WAVE;
+  };
+  // Load x is the first of its M0 group.
+  auto starts_group = [&](int x) __attribute__((always_inline)) { return (load_index(x) & 3) == 0; };
+  // M0 for the group that load x starts.
+  auto dma_base = [&](int kt_req, int x) __attribute__((always_inline)) {
+    uint32_t s = lds_base + (kt_req & (NS - 1)) * STAGE;
+    if (x < ATile::PER_WAVE) {
+      set_lds_dma_base(s + (wave * ATile::PER_WAVE + x) * 1024);
+    } else {
+      int y = x - ATile::PER_WAVE, bsel = y / BTile::PER_WAVE, i = y % BTile::PER_WAVE;
+      set_lds_dma_base(s + ATile::BYTES + bsel * BTile::BYTES + (wave * BTile::PER_WAVE + i) * 1024);
+    }
+  };
+  // The load itself (M0 must hold its group's base).  Tiles past the end are replaced by the last
+  // tile: the ring then always holds a full tile in flight, the redundant copies land in slots
+  // nobody reads again.
+  auto issue_one = [&](int kt_req, int x) __attribute__((always_inline)) {
+    int kt = kt_req < kt_total ? kt_req : kt_total - 1;
+    int seg = kt >= kt_seg ? 1 : 0;
+    int kk = kt - seg * kt_seg;
+    buffer_rsrc r;
+    uint32_t voff, soff;
+    if (x < ATile::PER_WAVE) {
+      r = seg ? ra[1] : ra[0];
+      voff = aoff[x];
+      soff = a_org + kk * a_step;
+    } else {
+      int y = x - ATile::PER_WAVE, bsel = y / BTile::PER_WAVE, i = y % BTile::PER_WAVE;
+      r = NB == 2 ? rb[bsel] : (seg ? rb[1] : rb[0]);
+      voff = boff[i];
+      soff = b_org + kk * b_step;
+    }
+    switch (load_index(x) & 3) {
+      case 0: load16_to_lds_at<0>(r, voff, soff); break;
+      case 1: load16_to_lds_at<1024>(r, voff, soff); break;
+      case 2: load16_to_lds_at<2048>(r, voff, soff); break;
+      default: load16_to_lds_at<3072>(r, voff, soff); break;
+    }
+  };
+
+  vec8 af[2][TM];  // A fragments: bank = step parity
+  vec8 bq[4];      // B fragment ring: entry = (step * G + group) % 4
+  auto fetch_a = [&](int bank, int i, int kt, int ks) __attribute__((always_inline)) {
+    const char* s = smem + (kt & (NS - 1)) * STAGE;
+    af[bank][i] = ATile::template frag_mi<MI>(s, wm * WTM + i * MI, ks, lane);
+  };
+  auto fetch_b = [&](int entry, int g, int kt, int ks) __attribute__((always_inline)) {
+    const char* s = smem + (kt & (NS - 1)) * STAGE;
+    const int bsel = g / TN, j = g % TN;
+    bq[entry] = BTile::template frag_mi<MI>(s + ATile::BYTES + bsel * BTile::BYTES,
+                                            wn * WTN + j * MI, ks, lane);
+  };
+
+  // One reduction tile.  NEXT: tile kt+1 exists.  The wavefront is alone on its SIMD: whatever
+  // issues between two MFMAs is hidden behind the matrix pipe, so every group is laid out as TM
+  // slots of {one MFMA; at most a couple of LDS fetches or one global->LDS load} and the
+  // scheduler is told to keep the slots.
+  auto tile_body = [&](int kt, auto next_c) __attribute__((always_inline)) {
+    constexpr bool NEXT = decltype(next_c)::value;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const bool last = ks == KSTEPS - 1;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool handover = last && g >= G - 2;  // groups that already work for tile kt+1
+        if (NEXT && last && g == G - 2) {
+          // No fetch addresses this tile's slot any more: wait until tile kt+1 has landed,
+          // barrier, then the slot can be refilled.
+          wait_vmem<0>();
+          __syncthreads();
+          if (LOAD_PHASE == 0) dma_base(kt + NS, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          acc[g][i] = mfma_mi<T, MI>(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
+          // --- B fragment of the group two ahead
+          if (i == 0) {
+            const int g2 = g + 2;
+            if (g2 < G) fetch_b((ks * G + g2) % 4, g2, kt, ks);
+            else if (!last) fetch_b(((ks + 1) * G + g2 - G) % 4, g2 - G, kt, ks + 1);
+            else if (NEXT) fetch_b((g2 - G) % 4, g2 - G, kt + 1, 0);
+          }
+          // --- A fragments of the next step: one per group, or all of them after the handover
+          if (!last) {
+            if (i == 1 && g < TM) fetch_a((ks + 1) & 1, g, kt, ks + 1);
+          } else if (NEXT && handover) {
+            const int h = (g - (G - 2)) * (TM / 2) + (i - 1);
+            if (i >= 1 && i <= TM / 2) fetch_a(0, h, kt + 1, 0);
+          }
+          // --- paced refill of the ring slot retired at the last barrier; slots are counted from
+          // that barrier, so a tile's loads start in the previous tile's handover groups.  Load x
+          // goes to slot x*LOAD_SLOTS + LOAD_PHASE, a new M0 one slot earlier.
+          if (NEXT) {
+            const int slot = handover ? (g - (G - 2)) * TM + i : HEAD_SLOTS + (ks * G + g) * TM + i;
+            const int lkt = handover ? kt + NS : kt + NS - 1;
+            if (slot % LOAD_SLOTS == LOAD_PHASE && slot / LOAD_SLOTS < L)
+              issue_one(lkt, slot / LOAD_SLOTS);
+            const int nx = (slot + 1) / LOAD_SLOTS;
+            if ((slot + 1) % LOAD_SLOTS == LOAD_PHASE && nx < L && starts_group(nx)) dma_base(lkt, nx);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  };
+
+  // Prologue: tile 0 .. NS-2 entirely, and of tile NS-1 the loads the handover groups would have
+  // issued (tile 0's own slots issue the rest); wait for tile 0.
+  constexpr int HEAD_LOADS = (HEAD_SLOTS - LOAD_PHASE + LOAD_SLOTS - 1) / LOAD_SLOTS;
+  constexpr int L_HEAD = HEAD_LOADS < L ? HEAD_LOADS : L;
+#pragma unroll
+  for (int x = 0; x < L; ++x) {
+    if (starts_group(x)) dma_base(0, x);
+    issue_one(0, x);
+  }
+#pragma unroll
+  for (int x = 0; x < L_HEAD; ++x) {
+    if (starts_group(x)) dma_base(1, x);
+    issue_one(1, x);
+  }
+  wait_vmem<L_HEAD>();
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i) fetch_a(0, i, 0, 0);
+  fetch_b(0, 0, 0, 0);
+  fetch_b(1, 1, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // Epilogue work items of a wavefront: MI-row slab i of its tile, then (row, 8-column group)
+  // items spread over the lanes.  What an epilogue reads from global memory is fetched
+  // PREFETCH_DEPTH items ahead, starting before the last reduction tile.
+  constexpr int ITEMS = MI * WTN / 8 / 64;  // items per lane and slab
+  constexpr int NITEMS = TM * ITEMS;
+  constexpr int PD = Epi::PREFETCH_DEPTH < NITEMS ? Epi::PREFETCH_DEPTH : NITEMS;
+  static_assert(MI * WTN / 8 % 64 == 0, "slab items must divide over the lanes");
+  auto item_pos = [&](int q, int& row, int& m, int& n, int& cg) __attribute__((always_inline)) {
+    int i = q / ITEMS, item = (q % ITEMS) * 64 + lane;
+    row = item / (WTN / 8);
+    cg = item % (WTN / 8);
+    m = m0 + wm * WTM + i * MI + row;
+    n = n0 + wn * WTN + cg * 8;
+  };
+  typename Epi::template Prefetch<8> pf[PD > 0 ? PD : 1];
+
+  int kt = 0;
+  for (; kt + 1 < kt_total; ++kt) tile_body(kt, std::true_type{});
+#pragma unroll
+  for (int q = 0; q < PD; ++q) {
+    int row, m, n, cg;
+    item_pos(q, row, m, n, cg);
+    Epi::template prefetch<8>(ea, m, n, pf[q]);
+  }
+  tile_body(kt, std::false_type{});
+  wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
+
+  // ---- epilogue: transpose MI-row slabs of the accumulators through LDS (fp32), then each lane
+  // owns 8 consecutive columns of one row.
+  __syncthreads();  // all wavefronts are done reading operand tiles
+  constexpr int ELD = Cfg::EPI_LD;
+  float* stg = (float*)(smem + wave * Cfg::EPI_WAVE_BYTES);
+  const int mrow = lane & (MI - 1), nsub = 4 * (lane / MI);
+  constexpr int NV = MI == 32 ? 4 : 1;  // 4-column vectors a lane holds per accumulator
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int b = g / TN, j = g % TN;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = acc[g][i][4 * v + r];
+        *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
+      }
+    }
+    // Same-wavefront LDS writes and reads are ordered; no barrier needed for a private slab.
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int q = i * ITEMS + it;
+      int row, m, n, cg;
+      item_pos(q, row, m, n, cg);
+      alignas(16) float v0[8], v1[8];
+      const float* p0 = stg + row * ELD + cg * 8;
+      *(f32x4*)v0 = *(const f32x4*)p0;
+      *(f32x4*)(v0 + 4) = *(const f32x4*)(p0 + 4);
+      if (NB == 2) {
+        const float* p1 = p0 + MI * ELD;
+        *(f32x4*)v1 = *(const f32x4*)p1;
+        *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
+      }
+      if (PD > 0) {
+        Epi::template apply<8>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
+        if (q + PD < NITEMS) {
+          int row2, m2, n2, cg2;
+          item_pos(q + PD, row2, m2, n2, cg2);
+          Epi::template prefetch<8>(ea, m2, n2, pf[q % (PD > 0 ? PD : 1)]);
+        }
+      } else {
+        Epi::template apply<8>(ea, m, n, v0, v1);
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64)
+    gemm_kernel_pipelined(GemmArgs ga, typename Epi::Args ea) {
+  gemm_pipelined_body<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(ga, ea, blockIdx.x, gridDim.x);
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64)
+    gemm_group_kernel_pipelined(GemmGroup<typename Epi::Args> grp) {
+  int g = 0;
+#pragma unroll
+  for (int i = 1; i < GEMM_GROUP_MAX; ++i)
+    if (i < grp.count && (int)blockIdx.x >= grp.first[i]) g = i;
+  GemmArgs ga = grp.ga[0];
+  typename Epi::Args ea = grp.ea[0];
+#pragma unroll
+  for (int i = 1; i < GEMM_GROUP_MAX; ++i)
+    if (g == i) { ga = grp.ga[i]; ea = grp.ea[i]; }
+  gemm_pipelined_body<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(
+      ga, ea, (int)blockIdx.x - grp.first[g], grp.first[g + 1] - grp.first[g]);
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
+  dim3 grid((ga.M / BM) * (ga.N / BN)), block(Cfg::NW * 64);
+  hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
+  return hipGetLastError();
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  auto kern = gemm_group_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
+  int total = 0;
+  for (int g = 0; g < grp.count; ++g) {
+    grp.first[g] = total;
+    total += (grp.ga[g].M / BM) * (grp.ga[g].N / BN);
+  }
+  for (int g = grp.count; g <= GEMM_GROUP_MAX; ++g) grp.first[g] = total;
+  hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);
+  return hipGetLastError();
+}
+
+}  // namespace gmlp

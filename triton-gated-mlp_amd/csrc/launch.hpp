@@ -1,7 +1,7 @@
 // Host-side launch interface between the C ABI (api.hip) and the kernel translation units.
 #pragma once
 #include "gemm.hpp"
-#include "gemm_v2.hpp"
+#include "gemm_tiles.hpp"
 
 namespace gmlp {
 

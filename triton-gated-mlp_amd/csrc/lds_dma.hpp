@@ -43,6 +43,28 @@ __device__ __forceinline__ void load16_to_lds(buffer_rsrc r, uint32_t voffset, u
   }
 }
 
+// The same transfer split in two, for loops where instruction issue is tight: M0 (the LDS base) is
+// written once for up to four loads, which then differ by the instruction's immediate offset
+// (0, 1024, 2048 or 3072).  The immediate is added to the LDS address AND to the global address,
+// so the caller passes a voffset that already has it subtracted (see DMA_BIAS in gemm_pipelined.hpp).
+// The compiler is not told that M0 stays live between the two statements; it has no use for M0 of
+// its own in kernels without indirect register indexing, message or GWS instructions.
+__device__ __forceinline__ void set_lds_dma_base(uint32_t lds_wave_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0"
+      :
+      : "s"(lds_wave_base)
+      : "memory");
+}
+template <int INST_OFF>
+__device__ __forceinline__ void load16_to_lds_at(buffer_rsrc r, uint32_t voffset, uint32_t soffset) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds"
+               :
+               : "v"(voffset), "s"(r), "s"(soffset), "n"(INST_OFF)
+               : "memory");
+}
+
 // The LDS write of a global->LDS load is complete when the wavefront's vector-memory counter has
 // drained past it; a workgroup barrier alone does not wait for it.  N = loads allowed in flight.
 template <int N>
