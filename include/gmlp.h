@@ -31,13 +31,31 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 1
+#define GMLP_ABI_VERSION 2
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
+/*
+ * Gate activation `act` of the hidden state H = act(G) ⊙ U.  The functions are those of the
+ * reference's hidden_act table (ACT2CLS / ACT_FWD, src/triton_gated_mlp/gated_mlp.py:17-37) with
+ * torch's default parameters: exact (erf) GELU, LeakyReLU slope 0.01; "swish" is GMLP_ACT_SILU and
+ * "no_act" is GMLP_ACT_IDENTITY.  The reference's fused kernels implement silu and no_act only
+ * (_act_fwd/_act_bwd, src/triton_gated_mlp/ops/act.py:5-22); derivatives here are the true ones
+ * (identity' = 1, relu'(0) = 0, leaky_relu'(0) = 0.01, as torch.autograd).
+ */
+enum gmlp_act {
+  GMLP_ACT_SILU = 0,
+  GMLP_ACT_GELU = 1,
+  GMLP_ACT_RELU = 2,
+  GMLP_ACT_LEAKY_RELU = 3,
+  GMLP_ACT_SIGMOID = 4,
+  GMLP_ACT_TANH = 5,
+  GMLP_ACT_IDENTITY = 6
+};
+
 enum gmlp_status {
   GMLP_OK = 0,
-  GMLP_EINVAL = -1, /* null pointer, bad dtype, bad dropout probability */
+  GMLP_EINVAL = -1, /* null pointer, bad dtype or act code, bad dropout probability */
   GMLP_ESHAPE = -2, /* shape not supported (see each entry point) */
   GMLP_EALIGN = -3, /* pointer not 16-byte aligned */
   GMLP_EHIP = -4    /* HIP runtime reported an error at launch */
@@ -53,7 +71,7 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
 
 /*
  * Hidden-state forward:  G = x·W_gateᵀ + b_gate,  U = x·W_upᵀ + b_up,
- *                        H = dropout(silu(G) ⊙ U).
+ *                        H = dropout(act(G) ⊙ U).
  * Replaces mlp_hidden_states_fwd + _fwd_kernel (src/triton_gated_mlp/ops/fwd.py:198-279, :72-166);
  * math of EagerGatedMLP.forward (src/triton_gated_mlp/gated_mlp.py:96) and eager_fwd (:105-128).
  * b_gate, b_up, g_save, u_save, mask_out may be NULL.  g_save/u_save [M,N] receive G and U
@@ -62,8 +80,8 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
  */
 int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
                     const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
-                    int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
-                    uint64_t offset, void* stream);
+                    int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p,
+                    uint64_t seed, uint64_t offset, void* stream);
 
 /*
  * Linear layer forward: out[M,C] = a[M,R]·w[C,R]ᵀ + bias[C]   (bias may be NULL).
@@ -75,22 +93,22 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
 
 /*
  * Backward through down_proj, dropout and the gating product in one GEMM:
- *   dH = dY·W_down ; dA = dH ⊙ keep/(1-p) ; dU = dA ⊙ silu(G) ; dG = dA ⊙ U ⊙ silu'(G).
+ *   dH = dY·W_down ; dA = dH ⊙ keep/(1-p) ; dU = dA ⊙ act(G) ; dG = dA ⊙ U ⊙ act'(G).
  * Replaces the autograd backward of down_proj plus _compute_quantities_for_bwd
  * (src/triton_gated_mlp/ops/bwd.py:89-211; closed form in gated_mlp.py:131-144).  g, u are the
  * tensors written by gmlp_gateup_fwd (g_save, u_save).  dg, du are [M,N].
  */
 int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
-                int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p, uint64_t seed,
                 uint64_t offset, void* stream);
 
 /*
  * Element-wise gating backward for callers that already hold dH (the reference's operator-level
- * backward receives grad_output = dH):  dU = dA ⊙ silu(G), dG = dA ⊙ U ⊙ silu'(G), dA as above.
+ * backward receives grad_output = dH):  dU = dA ⊙ act(G), dG = dA ⊙ U ⊙ act'(G), dA as above.
  * Replaces the epilogue of _compute_quantities_for_bwd (src/triton_gated_mlp/ops/bwd.py:196-211).
  */
 int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t M,
-                    int64_t N, int dtype, float dropout_p, uint64_t seed, uint64_t offset,
+                    int64_t N, int dtype, int act, float dropout_p, uint64_t seed, uint64_t offset,
                     void* stream);
 
 /*
@@ -129,7 +147,7 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
                 void* stream);
 
 /*
- * Skinny-M forward of the whole MLP (decode): y = (silu(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
+ * Skinny-M forward of the whole MLP (decode): y = (act(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
  * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch is [M,N] in dtype;
  * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
  * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
@@ -137,7 +155,7 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
  */
 int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                     const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
-                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype,
+                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype, int act,
                     void* stream);
 
 /* Writes the dropout keep mask (1 = keep) for an [M,N] tensor; the test oracle of the generator. */

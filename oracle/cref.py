@@ -35,7 +35,10 @@ def _p(a, t=ctypes.c_double):
     return None if a is None else a.ctypes.data_as(ctypes.POINTER(t))
 
 
-def forward(x, wg, bg, wu, bu, wd, bd, keep=None, p=0.0):
+ACT_CODES = {"silu": 0, "swish": 0, "gelu": 1, "relu": 2, "leaky_relu": 3, "sigmoid": 4, "tanh": 5, "no_act": 6}
+
+
+def forward(x, wg, bg, wu, bu, wd, bd, keep=None, p=0.0, act="silu"):
     x, wg, bg, wu, bu, wd, bd = map(_d, (x, wg, bg, wu, bu, wd, bd))
     M, K = x.shape
     N = wg.shape[0]
@@ -43,13 +46,14 @@ def forward(x, wg, bg, wu, bu, wd, bd, keep=None, p=0.0):
     G, U, H, Y = (np.empty((M, N)), np.empty((M, N)), np.empty((M, N)), np.empty((M, K)))
     lib().gmlp_ref_forward(
         _p(x), _p(wg), _p(bg), _p(wu), _p(bu), _p(wd), _p(bd), _p(keep, ctypes.c_uint8), ctypes.c_double(p),
-        ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), _p(G), _p(U), _p(H), _p(Y),
+        ctypes.c_int(ACT_CODES[act]), ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), _p(G), _p(U), _p(H),
+        _p(Y),
     )
     return {"G": G, "U": U, "H": H, "Y": Y}
 
 
-def backward(x, wg, bg, wu, bu, wd, bd, dY, keep=None, p=0.0):
-    f = forward(x, wg, bg, wu, bu, wd, bd, keep, p)
+def backward(x, wg, bg, wu, bu, wd, bd, dY, keep=None, p=0.0, act="silu"):
+    f = forward(x, wg, bg, wu, bu, wd, bd, keep, p, act)
     x, wg, wu, wd, dY = map(_d, (x, wg, wu, wd, dY))
     M, K = x.shape
     N = wg.shape[0]
@@ -59,7 +63,8 @@ def backward(x, wg, bg, wu, bu, wd, bd, dY, keep=None, p=0.0):
         "db_gate": np.empty(N), "db_up": np.empty(N), "db_down": np.empty(K),
     }
     lib().gmlp_ref_backward(
-        _p(x), _p(wg), _p(wu), _p(wd), _p(keep, ctypes.c_uint8), ctypes.c_double(p), _p(f["G"]), _p(f["U"]),
+        _p(x), _p(wg), _p(wu), _p(wd), _p(keep, ctypes.c_uint8), ctypes.c_double(p),
+        ctypes.c_int(ACT_CODES[act]), _p(f["G"]), _p(f["U"]),
         _p(f["H"]), _p(dY), ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), _p(out["dX"]),
         _p(out["dW_gate"]), _p(out["dW_up"]), _p(out["dW_down"]), _p(out["db_gate"]), _p(out["db_up"]),
         _p(out["db_down"]),

@@ -6,18 +6,22 @@ Restates the reference's eager module and closed forms (paths relative to the re
   backward   eager_bwd (hidden-state part)  src/triton_gated_mlp/gated_mlp.py:131-156
              _silu_op_bwd                   src/triton_gated_mlp/gated_mlp.py:40-43
              _silu_bwd / _compute_sigma     src/triton_gated_mlp/ops/act.py:28-45
+  activations ACT2CLS / ACT_FWD table       src/triton_gated_mlp/gated_mlp.py:17-37
 Dropout is expressed with an explicit keep mask D (nn.Dropout, gated_mlp.py:90,96, scales kept
-values by 1/(1-p)):  H = silu(G) * U * D / (1-p).
+values by 1/(1-p)):  H = act(G) * U * D / (1-p), act = silu unless stated.
 
 Pinned by tests/test_oracle.py: brute-force loops on tiny shapes, an independent NumPy fp64
 restatement, the C restatement in oracle/gated_mlp_ref.c, torch.autograd and gradcheck for the
-backward, known values of silu and silu', and algebraic special cases.  The reference holds no
+backward, known values of silu and silu', and algebraic special cases; the other activations and
+their closed-form derivatives (ACTS) against torch.nn.functional under torch.autograd, tabulated
+values and central differences.  The reference holds no
 stored vectors for this path (its tests compare fused against eager live), so nothing here is
 pinned against reference fixtures; no function depends on one.
 """
 
 from __future__ import annotations
 
+import math
 from typing import Dict, Optional
 
 import torch
@@ -33,6 +37,36 @@ def silu_grad(x: Tensor) -> Tensor:
     return s * (1 + x * (1 - s))
 
 
+def _gelu(x: Tensor) -> Tensor:
+    return 0.5 * x * (1 + torch.erf(x / math.sqrt(2.0)))
+
+
+def _gelu_grad(x: Tensor) -> Tensor:
+    return 0.5 * (1 + torch.erf(x / math.sqrt(2.0))) + x * torch.exp(-0.5 * x * x) / math.sqrt(2.0 * math.pi)
+
+
+def _sigmoid_grad(x: Tensor) -> Tensor:
+    s = torch.sigmoid(x)
+    return s * (1 - s)
+
+
+# name -> (act, act'): torch's defaults (erf GELU, LeakyReLU slope 0.01); at the kinks the
+# derivative is torch.autograd's (relu'(0) = 0, leaky_relu'(0) = 0.01).
+ACTS = {
+    "silu": (silu, silu_grad),
+    "swish": (silu, silu_grad),
+    "gelu": (_gelu, _gelu_grad),
+    "relu": (lambda x: torch.where(x > 0, x, torch.zeros_like(x)), lambda x: (x > 0).to(x.dtype)),
+    "leaky_relu": (
+        lambda x: torch.where(x > 0, x, 0.01 * x),
+        lambda x: torch.where(x > 0, torch.ones_like(x), torch.full_like(x, 0.01)),
+    ),
+    "sigmoid": (torch.sigmoid, _sigmoid_grad),
+    "tanh": (torch.tanh, lambda x: 1 - torch.tanh(x) ** 2),
+    "no_act": (lambda x: x, torch.ones_like),
+}
+
+
 def hidden_forward(
     x: Tensor,
     W_gate: Tensor,
@@ -41,6 +75,7 @@ def hidden_forward(
     b_up: Optional[Tensor],
     keep: Optional[Tensor] = None,
     p: float = 0.0,
+    act: str = "silu",
 ) -> Dict[str, Tensor]:
     G = x @ W_gate.T
     if b_gate is not None:
@@ -48,7 +83,7 @@ def hidden_forward(
     U = x @ W_up.T
     if b_up is not None:
         U = U + b_up
-    H = silu(G) * U
+    H = ACTS[act][0](G) * U
     if keep is not None and p > 0.0:
         H = H * keep.to(H.dtype) / (1.0 - p)
     return {"G": G, "U": U, "H": H}
@@ -64,9 +99,10 @@ def forward(
     b_down: Optional[Tensor],
     keep: Optional[Tensor] = None,
     p: float = 0.0,
+    act: str = "silu",
 ) -> Dict[str, Tensor]:
-    """Y = (silu(xW_gᵀ+b_g) ⊙ (xW_uᵀ+b_u) ⊙ D/(1-p)) W_dᵀ + b_d for 2-D x; returns Y and G, U, H."""
-    out = hidden_forward(x, W_gate, b_gate, W_up, b_up, keep, p)
+    """Y = (act(xW_gᵀ+b_g) ⊙ (xW_uᵀ+b_u) ⊙ D/(1-p)) W_dᵀ + b_d for 2-D x; returns Y and G, U, H."""
+    out = hidden_forward(x, W_gate, b_gate, W_up, b_up, keep, p, act)
     Y = out["H"] @ W_down.T
     if b_down is not None:
         Y = Y + b_down
@@ -75,12 +111,13 @@ def forward(
 
 
 def hidden_backward(
-    dH: Tensor, G: Tensor, U: Tensor, keep: Optional[Tensor] = None, p: float = 0.0
+    dH: Tensor, G: Tensor, U: Tensor, keep: Optional[Tensor] = None, p: float = 0.0, act: str = "silu"
 ) -> Dict[str, Tensor]:
     dA = dH
     if keep is not None and p > 0.0:
         dA = dH * keep.to(dH.dtype) / (1.0 - p)
-    return {"dU": dA * silu(G), "dG": dA * U * silu_grad(G)}
+    f, df = ACTS[act]
+    return {"dU": dA * f(G), "dG": dA * U * df(G)}
 
 
 def backward(
@@ -94,11 +131,12 @@ def backward(
     dY: Tensor,
     keep: Optional[Tensor] = None,
     p: float = 0.0,
+    act: str = "silu",
 ) -> Dict[str, Tensor]:
     """Closed-form gradients of `forward` for upstream gradient dY (all 2-D)."""
-    f = forward(x, W_gate, b_gate, W_up, b_up, W_down, b_down, keep, p)
+    f = forward(x, W_gate, b_gate, W_up, b_up, W_down, b_down, keep, p, act)
     dH = dY @ W_down
-    hb = hidden_backward(dH, f["G"], f["U"], keep, p)
+    hb = hidden_backward(dH, f["G"], f["U"], keep, p, act)
     dG, dU = hb["dG"], hb["dU"]
     out = {
         "dX": dU @ W_up + dG @ W_gate,

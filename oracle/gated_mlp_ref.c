@@ -6,6 +6,9 @@
  *   EagerGatedMLP.forward   src/triton_gated_mlp/gated_mlp.py:92-98
  *   eager_fwd / eager_bwd   src/triton_gated_mlp/gated_mlp.py:105-156
  *   silu' = s(1 + x(1-s))   src/triton_gated_mlp/gated_mlp.py:40-43, ops/act.py:42-45
+ *   hidden_act table        src/triton_gated_mlp/gated_mlp.py:17-37 (torch defaults: erf GELU,
+ *                           LeakyReLU slope 0.01); act codes 0..6 = silu, gelu, relu, leaky_relu,
+ *                           sigmoid, tanh, identity; derivatives at kinks as torch.autograd
  * with scalar loops in double precision, independent of torch and NumPy, so that the torch oracle
  * (oracle/eager.py) and the NumPy Philox (oracle/philox.py) each have a second implementation to
  * be checked against.  Layouts: row-major; W_gate, W_up [N,K]; W_down [K,N]; keep [M,N] uint8 or
@@ -18,11 +21,35 @@
 
 static double sigmoid(double v) { return 1.0 / (1.0 + exp(-v)); }
 
+static double act_fwd(int act, double v) {
+  switch (act) {
+    case 0: return v * sigmoid(v);
+    case 1: return 0.5 * v * (1.0 + erf(v / sqrt(2.0)));
+    case 2: return v > 0.0 ? v : 0.0;
+    case 3: return v > 0.0 ? v : 0.01 * v;
+    case 4: return sigmoid(v);
+    case 5: return tanh(v);
+    default: return v;
+  }
+}
+
+static double act_grad(int act, double v) {
+  switch (act) {
+    case 0: { double s = sigmoid(v); return s * (1.0 + v * (1.0 - s)); }
+    case 1: return 0.5 * (1.0 + erf(v / sqrt(2.0))) + v * exp(-0.5 * v * v) / sqrt(2.0 * M_PI);
+    case 2: return v > 0.0 ? 1.0 : 0.0;
+    case 3: return v > 0.0 ? 1.0 : 0.01;
+    case 4: { double s = sigmoid(v); return s * (1.0 - s); }
+    case 5: { double t = tanh(v); return 1.0 - t * t; }
+    default: return 1.0;
+  }
+}
+
 /* G, U, H: [M,N] outputs; Y: [M,K] output. */
 void gmlp_ref_forward(const double* x, const double* wg, const double* bg, const double* wu,
                       const double* bu, const double* wd, const double* bd, const uint8_t* keep,
-                      double p, int64_t M, int64_t K, int64_t N, double* G, double* U, double* H,
-                      double* Y) {
+                      double p, int act, int64_t M, int64_t K, int64_t N, double* G, double* U,
+                      double* H, double* Y) {
   for (int64_t m = 0; m < M; ++m)
     for (int64_t n = 0; n < N; ++n) {
       double g = bg ? bg[n] : 0.0, u = bu ? bu[n] : 0.0;
@@ -30,7 +57,7 @@ void gmlp_ref_forward(const double* x, const double* wg, const double* bg, const
         g += x[m * K + k] * wg[n * K + k];
         u += x[m * K + k] * wu[n * K + k];
       }
-      double h = g * sigmoid(g) * u;
+      double h = act_fwd(act, g) * u;
       if (keep && p > 0.0) h = keep[m * N + n] ? h / (1.0 - p) : 0.0;
       G[m * N + n] = g;
       U[m * N + n] = u;
@@ -48,7 +75,7 @@ void gmlp_ref_forward(const double* x, const double* wg, const double* bg, const
  * Outputs: dX [M,K], dWg [N,K], dWu [N,K], dWd [K,N], dbg [N], dbu [N], dbd [K] (bias outputs
  * may be NULL). */
 void gmlp_ref_backward(const double* x, const double* wg, const double* wu, const double* wd,
-                       const uint8_t* keep, double p, const double* G, const double* U,
+                       const uint8_t* keep, double p, int act, const double* G, const double* U,
                        const double* H, const double* dY, int64_t M, int64_t K, int64_t N,
                        double* dX, double* dWg, double* dWu, double* dWd, double* dbg, double* dbu,
                        double* dbd) {
@@ -59,9 +86,9 @@ void gmlp_ref_backward(const double* x, const double* wg, const double* wu, cons
       double dh = 0.0;
       for (int64_t k = 0; k < K; ++k) dh += dY[m * K + k] * wd[k * N + n];
       if (keep && p > 0.0) dh = keep[m * N + n] ? dh / (1.0 - p) : 0.0;
-      double g = G[m * N + n], s = sigmoid(g);
-      dU[m * N + n] = dh * g * s;
-      dG[m * N + n] = dh * U[m * N + n] * s * (1.0 + g * (1.0 - s));
+      double g = G[m * N + n];
+      dU[m * N + n] = dh * act_fwd(act, g);
+      dG[m * N + n] = dh * U[m * N + n] * act_grad(act, g);
     }
   for (int64_t m = 0; m < M; ++m)
     for (int64_t k = 0; k < K; ++k) {

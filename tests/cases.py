@@ -21,6 +21,7 @@ class Case:
     backward: bool = False
     seed: int = 0
     dropout_seed: int = 1234
+    act: str = "silu"
 
 
 CFG2 = Case("cfg2_llama7b_fwd", 4096, 4096, 11008, torch.float16)

@@ -50,9 +50,10 @@ def _run_module_case(c: Case):
     from triton_gated_mlp.ops import fwd as ops_fwd
 
     dev = _dev()
-    print(f"case {c.name}: M={c.M} K={c.K} N={c.N} dtype={c.dtype} bias={c.bias} p={c.p}", flush=True)
+    print(f"case {c.name}: M={c.M} K={c.K} N={c.N} dtype={c.dtype} bias={c.bias} p={c.p} act={c.act}", flush=True)
     t = make_inputs(c)
-    mlp = FusedGatedMLP(hidden_size=c.K, intermediate_size=c.N, bias=c.bias, dropout_p=c.p).to(dev).to(c.dtype)
+    mlp = FusedGatedMLP(hidden_size=c.K, intermediate_size=c.N, bias=c.bias, dropout_p=c.p, hidden_act=c.act)
+    mlp = mlp.to(dev).to(c.dtype)
     with torch.no_grad():
         mlp.gate_proj.weight.copy_(t["W_gate"])
         mlp.up_proj.weight.copy_(t["W_up"])
@@ -77,7 +78,9 @@ def _run_module_case(c: Case):
 
     o = _oracle_inputs(t)
     if not c.backward:
-        ref = oracle.forward(o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], keep, c.p)
+        ref = oracle.forward(
+            o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], keep, c.p, c.act
+        )
         _close("Y", y, ref["Y"])
         return
     grads_in = [x, mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight]
@@ -87,7 +90,7 @@ def _run_module_case(c: Case):
         names += ["db_gate", "db_up", "db_down"]
     grads = torch.autograd.grad(y, grads_in, grad_outputs=t["dY"].to(dev))
     ref = oracle.backward(
-        o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], o["dY"], keep, c.p
+        o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], o["dY"], keep, c.p, c.act
     )
     _close("Y", y, ref["Y"])
     for n, g in zip(names, grads):
@@ -127,6 +130,52 @@ def test_cfg5_fp16_decode_forward():
 )
 def test_small_shapes_forward_backward(M, K, N, bias, p, dtype):
     _run_module_case(Case(f"small_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=p, backward=True, seed=M + K + N))
+
+
+OTHER_ACTS = ["gelu", "relu", "leaky_relu", "sigmoid", "tanh", "no_act"]
+
+
+@pytest.mark.parametrize("act", OTHER_ACTS)
+def test_other_activations_forward_backward(act):
+    """hidden_act beyond silu (the reference's ACT_FWD table, src/triton_gated_mlp/gated_mlp.py:28-37):
+    full-tile kernels, bias, dropout; fp16."""
+    _run_module_case(Case(f"act_{act}", 384, 256, 640, torch.float16, bias=True, p=0.1, backward=True, seed=21, act=act))
+
+
+@pytest.mark.parametrize("act,dtype", [("gelu", torch.bfloat16), ("relu", torch.bfloat16), ("tanh", torch.float32)])
+def test_other_activations_ragged_shapes_and_dtypes(act, dtype):
+    _run_module_case(Case(f"act_{act}_ragged", 200, 136, 264, dtype, bias=True, p=0.25, backward=True, seed=22, act=act))
+
+
+@pytest.mark.parametrize("act", OTHER_ACTS)
+def test_other_activations_decode_path(act):
+    """M <= 16 in inference takes the weight-streaming kernels (both variants: K % 256 == 0 and not)."""
+    _run_module_case(Case(f"act_{act}_decode", 8, 1024, 1536, torch.float16, bias=True, seed=23, act=act))
+    _run_module_case(Case(f"act_{act}_decode_generic", 16, 96, 512, torch.float16, bias=False, seed=24, act=act))
+
+
+@pytest.mark.parametrize("act", ["gelu", "no_act"])
+def test_other_activations_operator_level(act):
+    """mlp_hidden_states_fwd / _bwd with act_fn, the reference operator signatures
+    (src/triton_gated_mlp/ops/fwd.py:198-206, ops/bwd.py:466-468).  The reference's no_act backward
+    multiplies by G instead of 1 (_act_bwd, ops/act.py:15-18); the true derivative is checked here."""
+    from triton_gated_mlp import mlp_hidden_states_bwd, mlp_hidden_states_fwd
+
+    dev = _dev()
+    c = Case(f"op_{act}", 256, 128, 384, torch.float16, backward=True, seed=25, act=act)
+    t = make_inputs(c)
+    g = torch.Generator().manual_seed(26)
+    dH = torch.randn(c.M, c.N, generator=g).to(c.dtype)
+    x, Wu, Wg = t["x"].to(dev), t["W_up"].to(dev), t["W_gate"].to(dev)
+    h = mlp_hidden_states_fwd(x, Wu, None, Wg, None, act, 0.0)
+    dx, dWu, dWg = mlp_hidden_states_bwd(x, Wu, Wg, dH.to(dev), act_fn=act)
+    o = _oracle_inputs(t)
+    f = oracle.hidden_forward(o["x"], o["W_gate"], None, o["W_up"], None, act=act)
+    hb = oracle.hidden_backward(dH.float(), f["G"], f["U"], act=act)
+    _close("H", h, f["H"])
+    _close("dX", dx, hb["dU"] @ o["W_up"] + hb["dG"] @ o["W_gate"])
+    _close("dW_up", dWu, hb["dU"].T @ o["x"], atol=ATOL * max(1.0, (hb["dU"].T @ o["x"]).abs().mean().item()))
+    _close("dW_gate", dWg, hb["dG"].T @ o["x"], atol=ATOL * max(1.0, (hb["dG"].T @ o["x"]).abs().mean().item()))
 
 
 def test_three_dimensional_input_matches_flattened():

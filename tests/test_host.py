@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"libgmlp.so does not export {name}"
     assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
-    assert lib.gmlp_abi_version() == 1
+    assert lib.gmlp_abi_version() == 2
 
 
 def _buf(nbytes=4096):
@@ -47,23 +47,27 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None) == -1 and "NULL" in err()
     # bad dtype; float32 is not available for the skinny-M kernels
     assert lib.gmlp_linear_fwd(a, a, None, a, 8, 8, 8, 7, None) == -1 and "dtype" in err()
-    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 256, 2, None) == -2
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 256, 2, 0, None) == -2
     # shape: K not a multiple of 8, M < 1
     assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None) == -2 and "multiple of 8" in err()
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0.0, 0, 0, None) == -2
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0, 0.0, 0, 0, None) == -2
     # alignment
     assert lib.gmlp_linear_fwd(a + 2, a, None, a, 8, 8, 8, 0, None) == -3 and "aligned" in err()
     # dropout probability outside [0, 1)
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 1.0, 0, 0, None) == -1
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, -0.1, 0, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, 1.0, 0, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, -0.1, 0, 0, None) == -1
     assert lib.gmlp_dropout_mask(a, 8, 8, float("nan"), 0, 0, None) == -1
+    # activation code outside the GMLP_ACT_* range
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 7, 0.0, 0, 0, None) == -1
+    assert "act" in err()
+    assert lib.gmlp_gating_bwd(a, a, a, a, a, 8, 8, 0, -1, 0.0, 0, 0, None) == -1
     # decode limits
-    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 17, 256, 256, 0, None) == -2 and "16" in err()
-    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 40, 256, 0, None) == -2
-    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 128, 0, None) == -2
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 17, 256, 256, 0, 0, None) == -2 and "16" in err()
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 40, 256, 0, 0, None) == -2
+    assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 128, 0, 0, None) == -2
     for fn, args in [
-        (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0.0, 0, 0, None)),
-        (lib.gmlp_gating_bwd, (a, a, a, a, None, 8, 8, 0, 0.0, 0, 0, None)),
+        (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0, 0.0, 0, 0, None)),
+        (lib.gmlp_gating_bwd, (a, a, a, a, None, 8, 8, 0, 0, 0.0, 0, 0, None)),
         (lib.gmlp_dx_bwd, (a, a, a, a, None, 8, 8, 8, 0, None)),
         (lib.gmlp_dw_bwd, (a, None, a, 8, 8, 8, 0, None)),
         (lib.gmlp_colsum, (a, a, None, 8, 8, 0, None)),
@@ -106,8 +110,15 @@ def test_module_surface_matches_reference():
     assert [n for n, _ in FusedGatedMLP(bias=False).named_parameters()] == [
         "gate_proj.weight", "up_proj.weight", "down_proj.weight"]
     assert set(ACT_FWD) >= {"silu", "swish", "gelu", "relu", "no_act"}
+    # every activation of the reference's table constructs; an unknown name fails like its dict lookup
+    for act in ACT_FWD:
+        assert FusedGatedMLP(hidden_act=act).act_fn == act
+        assert _cabi.act_code(act) in range(7)
+    assert _cabi.act_code("swish") == _cabi.act_code("silu") == 0 and _cabi.act_code("no_act") == 6
+    with pytest.raises(KeyError):
+        FusedGatedMLP(hidden_act="softplus")
     with pytest.raises(NotImplementedError):
-        FusedGatedMLP(hidden_act="gelu")
+        _cabi.act_code("softplus")
     for name in ("EagerGatedMLP", "FusedGatedMLP", "FusedGatedMLPFunction", "mlp_hidden_states_fwd",
                  "mlp_hidden_states_bwd", "eager_fwd", "eager_bwd", "ACT_FWD"):
         assert hasattr(tgm.gated_mlp, name)
@@ -165,4 +176,4 @@ def test_operator_shape_validation_happens_before_device_checks():
     with pytest.raises(ValueError):
         validate_dimensions(x, W, torch.zeros(7), W, None)
     with pytest.raises(NotImplementedError):
-        tgm.mlp_hidden_states_fwd(x, W, None, W, None, "gelu", 0.0)
+        tgm.mlp_hidden_states_fwd(x, W, None, W, None, "softplus", 0.0)

@@ -132,6 +132,68 @@ def test_silu_known_values_and_derivative():
     assert torch.allclose(oracle.silu_grad(xs), ga, atol=1e-12)
 
 
+TORCH_ACT = {
+    "silu": torch.nn.functional.silu,
+    "swish": torch.nn.functional.silu,
+    "gelu": torch.nn.functional.gelu,
+    "relu": torch.nn.functional.relu,
+    "leaky_relu": torch.nn.functional.leaky_relu,
+    "sigmoid": torch.sigmoid,
+    "tanh": torch.tanh,
+    "no_act": lambda v: v,
+}
+# act(1), act(-1), act'(1), act'(-1) from the definitions: Phi(1) = 0.841344746..., phi(1) = 0.241970724...
+ACT_TABLE = {
+    "gelu": (0.8413447460685429, -0.15865525393145707, 1.0833154705876864, -0.08331547058768629),
+    "relu": (1.0, 0.0, 1.0, 0.0),
+    "leaky_relu": (1.0, -0.01, 1.0, 0.01),
+    "sigmoid": (0.7310585786300049, 0.2689414213699951, 0.19661193324148185, 0.19661193324148185),
+    "tanh": (0.7615941559557649, -0.7615941559557649, 0.41997434161402614, 0.41997434161402614),
+    "no_act": (1.0, -1.0, 1.0, 1.0),
+}
+
+
+@pytest.mark.parametrize("act", sorted(TORCH_ACT))
+def test_activation_table_against_torch_autograd_and_central_differences(act):
+    f, df = oracle.ACTS[act]
+    xs = torch.cat([torch.linspace(-6, 6, 101, dtype=torch.float64), torch.tensor([0.0], dtype=torch.float64)])
+    xa = xs.clone().requires_grad_(True)
+    ya = TORCH_ACT[act](xa)
+    (ga,) = torch.autograd.grad(ya.sum(), xa)
+    assert torch.allclose(f(xs), ya.detach(), atol=1e-12), "forward differs from torch.nn.functional"
+    assert torch.allclose(df(xs), ga, atol=1e-12), "derivative differs from torch.autograd (kinks included)"
+    smooth = xs[xs.abs() > 1e-3]  # central differences away from the kink at 0
+    h = 1e-6
+    assert torch.allclose(df(smooth), (f(smooth + h) - f(smooth - h)) / (2 * h), atol=1e-8)
+    if act in ACT_TABLE:
+        one = torch.tensor([1.0, -1.0], dtype=torch.float64)
+        exp = torch.tensor(ACT_TABLE[act], dtype=torch.float64)
+        assert torch.allclose(torch.cat([f(one), df(one)]), exp, atol=1e-12)
+
+
+@pytest.mark.parametrize("act", ["gelu", "relu", "leaky_relu", "sigmoid", "tanh", "no_act"])
+def test_other_activations_full_path_against_autograd_and_c(act):
+    t = _rand_problem(5, 4, 6, True, seed=11)
+    p = 0.25
+    leaves = {k: v.clone().requires_grad_(True) for k, v in t.items() if k not in ("dY", "keep")}
+    g = torch.nn.functional.linear(leaves["x"], leaves["W_gate"], leaves["b_gate"])
+    u = torch.nn.functional.linear(leaves["x"], leaves["W_up"], leaves["b_up"])
+    h = TORCH_ACT[act](g) * u * t["keep"].to(torch.float64) / (1 - p)
+    y = torch.nn.functional.linear(h, leaves["W_down"], leaves["b_down"])
+    names = list(leaves)
+    grads = torch.autograd.grad(y, [leaves[k] for k in names], grad_outputs=t["dY"])
+    got = oracle.backward(*_args(t), t["dY"], keep=t["keep"], p=p, act=act)
+    key = {"x": "dX", "W_gate": "dW_gate", "W_up": "dW_up", "W_down": "dW_down", "b_gate": "db_gate", "b_up": "db_up",
+           "b_down": "db_down"}
+    assert torch.allclose(got["Y"], y.detach(), rtol=1e-12, atol=1e-12)
+    for n, gr in zip(names, grads):
+        assert torch.allclose(got[key[n]], gr, rtol=1e-11, atol=1e-11), n
+    x, Wg, bg, Wu, bu, Wd, bd = [v.numpy() for v in _args(t)]
+    c = cref.backward(x, Wg, bg, Wu, bu, Wd, bd, t["dY"].numpy(), keep=t["keep"].numpy(), p=p, act=act)
+    for k in ("Y", "H", "dX", "dW_gate", "dW_up", "dW_down", "db_gate", "db_up", "db_down"):
+        assert np.allclose(c[k], got[k].numpy(), rtol=1e-11, atol=1e-11), k
+
+
 def test_algebraic_special_cases():
     t = _rand_problem(6, 5, 7, True, seed=4)
     a = list(_args(t))

@@ -32,6 +32,16 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
   if ((d) != GMLP_F16 && (d) != GMLP_BF16 && (d) != GMLP_F32)                       \
   return fail(GMLP_EINVAL, "%s: dtype %d is not GMLP_F16/GMLP_BF16/GMLP_F32", __func__, (int)(d))
 
+#define GMLP_REQUIRE_ACT(a)                                                         \
+  if ((a) < 0 || (a) >= gmlp::ACT_COUNT)                                            \
+  return fail(GMLP_EINVAL, "%s: act %d is not one of the GMLP_ACT_* codes", __func__, (int)(a))
+
+static_assert((int)GMLP_ACT_SILU == (int)gmlp::ACT_SILU && (int)GMLP_ACT_GELU == (int)gmlp::ACT_GELU &&
+                  (int)GMLP_ACT_RELU == (int)gmlp::ACT_RELU && (int)GMLP_ACT_LEAKY_RELU == (int)gmlp::ACT_LEAKY_RELU &&
+                  (int)GMLP_ACT_SIGMOID == (int)gmlp::ACT_SIGMOID && (int)GMLP_ACT_TANH == (int)gmlp::ACT_TANH &&
+                  (int)GMLP_ACT_IDENTITY == (int)gmlp::ACT_IDENTITY && gmlp::ACT_COUNT == 7,
+              "device activation codes are the public ones");
+
 const int64_t kMaxDim = (int64_t)1 << 30;
 
 int check_dims(const char* fn, int64_t M, int64_t K, int64_t N) {
@@ -105,11 +115,12 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) 
 
 int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
                     const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
-                    int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
-                    uint64_t offset, void* stream) {
+                    int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p,
+                    uint64_t seed, uint64_t offset, void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(x); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up); GMLP_REQUIRE_PTR(h);
   GMLP_REQUIRE_DTYPE(dtype);
+  GMLP_REQUIRE_ACT(act);
   DropoutParams d;
   if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
   if (int rc = check_dims(__func__, M, K, N)) return rc;
@@ -128,7 +139,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
     typename EpiGateUp<T>::Args ea = {(T*)h, (T*)g_save, (T*)u_save, mask_out, (const T*)b_gate,
-                                      (const T*)b_up, (int)N, d};
+                                      (const T*)b_up, (int)N, act, d};
     return launch_gateup<T>(tc, ga, ea, s);
   });
   return hip_result(__func__, e);
@@ -160,12 +171,13 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
 }
 
 int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
-                int64_t M, int64_t K, int64_t N, int dtype, float dropout_p, uint64_t seed,
+                int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p, uint64_t seed,
                 uint64_t offset, void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(dy); GMLP_REQUIRE_PTR(w_down); GMLP_REQUIRE_PTR(g); GMLP_REQUIRE_PTR(u);
   GMLP_REQUIRE_PTR(dg); GMLP_REQUIRE_PTR(du);
   GMLP_REQUIRE_DTYPE(dtype);
+  GMLP_REQUIRE_ACT(act);
   DropoutParams d;
   if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
   if (int rc = check_dims(__func__, M, K, N)) return rc;
@@ -183,19 +195,20 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
-    typename EpiDh<T>::Args ea = {(const T*)g, (const T*)u, (T*)dg, (T*)du, (int)N, d};
+    typename EpiDh<T>::Args ea = {(const T*)g, (const T*)u, (T*)dg, (T*)du, (int)N, act, d};
     return launch_dh<T>(tc, ga, ea, s);
   });
   return hip_result(__func__, e);
 }
 
 int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t M,
-                    int64_t N, int dtype, float dropout_p, uint64_t seed, uint64_t offset,
+                    int64_t N, int dtype, int act, float dropout_p, uint64_t seed, uint64_t offset,
                     void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(dh); GMLP_REQUIRE_PTR(g); GMLP_REQUIRE_PTR(u); GMLP_REQUIRE_PTR(dg);
   GMLP_REQUIRE_PTR(du);
   GMLP_REQUIRE_DTYPE(dtype);
+  GMLP_REQUIRE_ACT(act);
   DropoutParams d;
   if (int rc = make_dropout(__func__, dropout_p, seed, offset, &d)) return rc;
   if (int rc = check_dims(__func__, M, 8, N)) return rc;
@@ -205,7 +218,7 @@ int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
-    return launch_gating_bwd<T>((const T*)dh, (const T*)g, (const T*)u, (T*)dg, (T*)du, M, N, d, s);
+    return launch_gating_bwd<T>((const T*)dh, (const T*)g, (const T*)u, (T*)dg, (T*)du, M, N, act, d, s);
   });
   return hip_result(__func__, e);
 }
@@ -330,13 +343,14 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
 
 int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                     const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
-                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype,
+                    void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype, int act,
                     void* stream) {
   using namespace gmlp;
   (void)workspace;
   GMLP_REQUIRE_PTR(x); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up); GMLP_REQUIRE_PTR(w_down);
   GMLP_REQUIRE_PTR(h_scratch); GMLP_REQUIRE_PTR(y);
   GMLP_REQUIRE_DTYPE(dtype);
+  GMLP_REQUIRE_ACT(act);
   if (int rc = check_dims(__func__, M, K, N)) return rc;
   if (dtype == GMLP_F32) return fail(GMLP_ESHAPE, "%s: float32 is not supported by the skinny-M kernels", __func__);
   if (M > 16) return fail(GMLP_ESHAPE, "%s: M = %lld exceeds the skinny-M limit of 16", __func__, (long long)M);
@@ -350,11 +364,11 @@ int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const v
       dtype == GMLP_F16
           ? launch_decode<f16>((const f16*)x, (const f16*)w_gate, (const f16*)w_up, (const f16*)w_down,
                                (const f16*)b_gate, (const f16*)b_up, (const f16*)b_down,
-                               (f16*)h_scratch, (f16*)y, (int)M, (int)K, (int)N, s)
+                               (f16*)h_scratch, (f16*)y, (int)M, (int)K, (int)N, act, s)
           : launch_decode<bf16>((const bf16*)x, (const bf16*)w_gate, (const bf16*)w_up,
                                 (const bf16*)w_down, (const bf16*)b_gate, (const bf16*)b_up,
                                 (const bf16*)b_down, (bf16*)h_scratch, (bf16*)y, (int)M, (int)K,
-                                (int)N, s);
+                                (int)N, act, s);
   return hip_result(__func__, e);
 }
 

@@ -7,33 +7,35 @@ namespace gmlp {
 template <typename T>
 __global__ void __launch_bounds__(256)
     gating_bwd_kernel(const T* __restrict__ dh, const T* __restrict__ g, const T* __restrict__ u,
-                      T* __restrict__ dg, T* __restrict__ du, size_t n8, DropoutParams d) {
+                      T* __restrict__ dg, T* __restrict__ du, size_t n8, int act,
+                      DropoutParams d) {
   size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
     size_t e = i * 8;
     float v[8];
     load_w<T, 8>(dh + e, v);
-    gating_bwd_w<T, 8>(d, e, v, g, u, dg, du);
+    gating_bwd_w<T, 8>(act, d, e, v, g, u, dg, du);
   }
 }
 
 template <typename T>
 hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
-                             const DropoutParams& d, hipStream_t s) {
+                             int act, const DropoutParams& d, hipStream_t s) {
   size_t n8 = (size_t)M * N / 8;
   if (n8 == 0) return hipSuccess;
   size_t blocks = (n8 + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
   hipLaunchKernelGGL(gating_bwd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, dh, g, u, dg, du,
-                     n8, d);
+                     n8, act, d);
   return hipGetLastError();
 }
 template hipError_t launch_gating_bwd<f16>(const f16*, const f16*, const f16*, f16*, f16*, int64_t,
-                                           int64_t, const DropoutParams&, hipStream_t);
+                                           int64_t, int, const DropoutParams&, hipStream_t);
 template hipError_t launch_gating_bwd<bf16>(const bf16*, const bf16*, const bf16*, bf16*, bf16*,
-                                            int64_t, int64_t, const DropoutParams&, hipStream_t);
+                                            int64_t, int64_t, int, const DropoutParams&,
+                                            hipStream_t);
 template hipError_t launch_gating_bwd<float>(const float*, const float*, const float*, float*,
-                                             float*, int64_t, int64_t, const DropoutParams&,
+                                             float*, int64_t, int64_t, int, const DropoutParams&,
                                              hipStream_t);
 
 // Column sums in two fixed-order stages: COLSUM_SPLITS row ranges -> fp32 partials -> total.

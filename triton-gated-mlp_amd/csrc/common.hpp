@@ -69,6 +69,122 @@ __device__ __forceinline__ float silu_grad_f32(float x) {
   return s * (1.0f + x * (1.0f - s));
 }
 
+// Gate activations.  The codes are the GMLP_ACT_* values of the C interface; the functions are the
+// ones the reference's eager module offers for hidden_act (ACT2CLS / ACT_FWD,
+// src/triton_gated_mlp/gated_mlp.py:17-37) with torch's default parameters: exact (erf) GELU,
+// LeakyReLU slope 0.01.  Derivatives follow torch.autograd at the kinks: relu'(0) = 0,
+// leaky_relu'(0) = 0.01.  Everything is evaluated in fp32.
+enum Act : int {
+  ACT_SILU = 0,
+  ACT_GELU = 1,
+  ACT_RELU = 2,
+  ACT_LEAKY_RELU = 3,
+  ACT_SIGMOID = 4,
+  ACT_TANH = 5,
+  ACT_IDENTITY = 6,
+  ACT_COUNT = 7
+};
+constexpr float LEAKY_SLOPE = 0.01f;
+
+// y[r] = act(x[r]) for W values; `act` is uniform over the wavefront, so the switch is a scalar
+// branch taken once per call.  ACT >= 0 fixes the activation at compile time (`act` is ignored and
+// the other cases are not emitted); ACT_RUNTIME keeps the switch.
+constexpr int ACT_RUNTIME = -1;
+template <int W, int ACT = ACT_RUNTIME>
+__device__ __forceinline__ void act_fwd_w(int act, const float* x, float* y) {
+  switch (ACT >= 0 ? ACT : act) {
+    case ACT_SILU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = silu_f32(x[r]);
+      break;
+    case ACT_GELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = 0.5f * x[r] * (1.0f + erff(x[r] * 0.70710678118654752f));
+      break;
+    case ACT_RELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = x[r] < 0.f ? 0.f : x[r];
+      break;
+    case ACT_LEAKY_RELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = x[r] < 0.f ? LEAKY_SLOPE * x[r] : x[r];
+      break;
+    case ACT_SIGMOID:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = sigmoid_f32(x[r]);
+      break;
+    case ACT_TANH:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = tanhf(x[r]);
+      break;
+    default:
+#pragma unroll
+      for (int r = 0; r < W; ++r) y[r] = x[r];
+      break;
+  }
+}
+
+// y[r] = act(x[r]) and d[r] = act'(x[r]).
+template <int W, int ACT = ACT_RUNTIME>
+__device__ __forceinline__ void act_fwd_grad_w(int act, const float* x, float* y, float* d) {
+  switch (ACT >= 0 ? ACT : act) {
+    case ACT_SILU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        float s = sigmoid_f32(x[r]);
+        y[r] = x[r] * s;
+        d[r] = s * (1.0f + x[r] * (1.0f - s));
+      }
+      break;
+    case ACT_GELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        float cdf = 0.5f * (1.0f + erff(x[r] * 0.70710678118654752f));
+        float pdf = 0.39894228040143268f * __expf(-0.5f * x[r] * x[r]);
+        y[r] = x[r] * cdf;
+        d[r] = cdf + x[r] * pdf;
+      }
+      break;
+    case ACT_RELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        y[r] = x[r] < 0.f ? 0.f : x[r];
+        d[r] = x[r] > 0.f ? 1.f : 0.f;
+      }
+      break;
+    case ACT_LEAKY_RELU:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        y[r] = x[r] < 0.f ? LEAKY_SLOPE * x[r] : x[r];
+        d[r] = x[r] > 0.f ? 1.f : LEAKY_SLOPE;
+      }
+      break;
+    case ACT_SIGMOID:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        float s = sigmoid_f32(x[r]);
+        y[r] = s;
+        d[r] = s * (1.0f - s);
+      }
+      break;
+    case ACT_TANH:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        float t = tanhf(x[r]);
+        y[r] = t;
+        d[r] = 1.0f - t * t;
+      }
+      break;
+    default:
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        y[r] = x[r];
+        d[r] = 1.0f;
+      }
+      break;
+  }
+}
+
 // Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
 __host__ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2,
                                                         uint32_t c3, uint32_t k0, uint32_t k1,

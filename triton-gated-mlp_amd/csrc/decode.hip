@@ -1,7 +1,7 @@
 // Skinny-M (M <= 16) forward of the whole gated MLP: the three weight matrices are streamed from
 // HBM exactly once; the token block x (and the hidden block H) is small enough to stay in L2.
 //
-// Phase 1  H[m,n] = silu(x·W_gateᵀ + b_g) * (x·W_upᵀ + b_u)
+// Phase 1  H[m,n] = act(x·W_gateᵀ + b_g) * (x·W_upᵀ + b_u)
 //   one wavefront per block of 16 hidden columns n; v_mfma_f32_16x16x32 with the 16 weight rows as
 //   the instruction's A operand and the 16 token rows as its B operand, so a lane accumulates
 //   4 consecutive n of one token row.  Each lane loads its weight fragments straight from global
@@ -42,7 +42,8 @@ template <typename T>
 __global__ void __launch_bounds__(256)
     decode_gateup_kernel(const T* __restrict__ x, const T* __restrict__ wg,
                          const T* __restrict__ wu, const T* __restrict__ bg,
-                         const T* __restrict__ bu, T* __restrict__ h, int M, int K, int N) {
+                         const T* __restrict__ bu, T* __restrict__ h, int M, int K, int N,
+                         int act) {
   typedef typename Traits<T>::vec8 vec8;
   constexpr int U = DEC_UNROLL;
   const int lane = threadIdx.x & 63;
@@ -117,8 +118,9 @@ __global__ void __launch_bounds__(256)
     for (int r = 0; r < 4; ++r) { g[r] = accg[r]; u[r] = accu[r]; }
     if (bg) add_w<T, 4>(bg + n, g);
     if (bu) add_w<T, 4>(bu + n, u);
+    act_fwd_w<4>(act, g, hv);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) hv[r] = silu_f32(g[r]) * u[r];
+    for (int r = 0; r < 4; ++r) hv[r] *= u[r];
     store_w<T, 4>(h + (size_t)r16 * N + n, hv);
   }
 }
@@ -199,12 +201,13 @@ __global__ void __launch_bounds__(DEC_SPLIT * 64)
 
 template <typename T>
 hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
-                         const T* bu, const T* bd, T* h, T* y, int M, int K, int N, hipStream_t s) {
+                         const T* bu, const T* bd, T* h, T* y, int M, int K, int N, int act,
+                         hipStream_t s) {
   if (decode_stream_supported(M, K, N))
-    return launch_decode_stream<T>(x, wg, wu, wd, bg, bu, bd, h, y, M, K, N, s);
+    return launch_decode_stream<T>(x, wg, wu, wd, bg, bu, bd, h, y, M, K, N, act, s);
   int nblocks = N / 16;
   hipLaunchKernelGGL(decode_gateup_kernel<T>, dim3((nblocks + 3) / 4), dim3(256), 0, s, x, wg, wu,
-                     bg, bu, h, M, K, N);
+                     bg, bu, h, M, K, N, act);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(decode_down_kernel<T>, dim3(K / 16), dim3(DEC_SPLIT * 64), 0, s, h, wd, bd, y,
@@ -213,10 +216,10 @@ hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, cons
 }
 
 template hipError_t launch_decode<f16>(const f16*, const f16*, const f16*, const f16*, const f16*,
-                                       const f16*, const f16*, f16*, f16*, int, int, int,
+                                       const f16*, const f16*, f16*, f16*, int, int, int, int,
                                        hipStream_t);
 template hipError_t launch_decode<bf16>(const bf16*, const bf16*, const bf16*, const bf16*,
                                         const bf16*, const bf16*, const bf16*, bf16*, bf16*, int,
-                                        int, int, hipStream_t);
+                                        int, int, int, hipStream_t);
 
 }  // namespace gmlp

@@ -13,7 +13,7 @@
 // The stream of stages runs on across block boundaries, so the ring never drains; loads past the
 // end re-fetch the last stage into a free slot, which keeps the in-flight count constant.
 //
-//   GATED:   H[m, r] = silu(x.W_gate[r] + b_gate[r]) * (x.W_up[r] + b_up[r])     (r over N)
+//   GATED:   H[m, r] = act(x.W_gate[r] + b_gate[r]) * (x.W_up[r] + b_up[r])      (r over N)
 //   !GATED:  Y[m, r] = H.W_down[r] + b_down[r]                                   (r over K)
 //
 // LDS layout of a slot: 2 regions of 16 rows x 512 bytes; the 16-byte chunk c of row r is
@@ -55,6 +55,7 @@ struct StreamArgs {
   const void* bias[2];
   void* out;          // [M, ldo]
   int M, R, red, ldx, ldo;
+  int act;            // Act code (GATED only)
 };
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -197,8 +198,9 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
             }
             if (GATED) {
               float res[4];
+              act_fwd_w<4>(a.act, v[0], res);
 #pragma unroll
-              for (int r = 0; r < 4; ++r) res[r] = silu_f32(v[0][r]) * v[1][r];
+              for (int r = 0; r < 4; ++r) res[r] *= v[1][r];
               store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
             } else {
               store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, v[0]);
@@ -234,23 +236,23 @@ bool decode_stream_supported(int M, int K, int N) {
 template <typename T>
 hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
                                 const T* bu, const T* bd, T* h, T* y, int M, int K, int N,
-                                hipStream_t s) {
+                                int act, hipStream_t s) {
   int dev = 0, num_cu = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   if (hipError_t e = hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev)) return e;
   if (num_cu <= 0) num_cu = 256;
-  StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N};
+  StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act};
   hipError_t e = launch_stream<T, true>(a1, num_cu, s);
   if (e != hipSuccess) return e;
-  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K};
+  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY};
   return launch_stream<T, false>(a2, num_cu, s);
 }
 
 template hipError_t launch_decode_stream<f16>(const f16*, const f16*, const f16*, const f16*,
                                               const f16*, const f16*, const f16*, f16*, f16*, int,
-                                              int, int, hipStream_t);
+                                              int, int, int, hipStream_t);
 template hipError_t launch_decode_stream<bf16>(const bf16*, const bf16*, const bf16*, const bf16*,
                                                const bf16*, const bf16*, const bf16*, bf16*, bf16*,
-                                               int, int, int, hipStream_t);
+                                               int, int, int, int, hipStream_t);
 
 }  // namespace gmlp

@@ -285,20 +285,21 @@ struct EpiStore {
     if (a.bias) add_w<T, W>(a.bias + n, v);
     store_w<T, W>(a.out + (size_t)m * a.ldc + n, v);
   }
-  // Nothing worth fetching ahead of time (see EpiDh).
+  // Nothing worth fetching ahead of time (see EpiDh), no activation to specialise on.
   static constexpr int PREFETCH_DEPTH = 0;
+  static constexpr bool HAS_ACT = false;
   template <int W>
   struct Prefetch {};
   template <int W>
   static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
-  template <int W>
+  template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float* w,
                                                const Prefetch<W>&) {
     apply<W>(a, m, n, v, w);
   }
 };
 
-// G = acc0 + b_gate, U = acc1 + b_up, H = dropout(silu(G) * U)
+// G = acc0 + b_gate, U = acc1 + b_up, H = dropout(act(G) * U)
 template <typename T>
 struct EpiGateUp {
   struct Args {
@@ -309,16 +310,22 @@ struct EpiGateUp {
     const T* b_gate;    // nullable
     const T* b_up;      // nullable
     int ldc;
+    int act;            // Act code
     DropoutParams drop;
   };
-  template <int W>
+  // ACT: activation fixed at compile time, or ACT_RUNTIME to read a.act.  A kernel whose epilogue
+  // is unrolled many times instantiates both and branches once, so that the usual SiLU path stays
+  // as compact as if it were the only one (HAS_ACT tells it that the choice exists).
+  static constexpr bool HAS_ACT = true;
+  template <int W, int ACT = ACT_RUNTIME>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* g, float* u) {
     if (a.b_gate) add_w<T, W>(a.b_gate + n, g);
     if (a.b_up) add_w<T, W>(a.b_up + n, u);
     size_t e = (size_t)m * a.ldc + n;
     float h[W];
+    act_fwd_w<W, ACT>(a.act, g, h);
 #pragma unroll
-    for (int r = 0; r < W; ++r) h[r] = silu_f32(g[r]) * u[r];
+    for (int r = 0; r < W; ++r) h[r] *= u[r];
     if (a.drop.enabled) {
       bool keep[W];
       keep_w<W>(a.drop, e, keep);
@@ -346,16 +353,16 @@ struct EpiGateUp {
   struct Prefetch {};
   template <int W>
   static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
-  template <int W>
+  template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* g, float* u,
                                                const Prefetch<W>&) {
-    apply<W>(a, m, n, g, u);
+    apply<W, ACT>(a, m, n, g, u);
   }
 };
 
-// Gating backward on W consecutive elements: dA = dH*keep/(1-p); dU = dA*silu(G); dG = dA*U*silu'(G)
-template <typename T, int W>
-__device__ __forceinline__ void gating_bwd_core(const DropoutParams& drop, size_t e, float* dh,
+// Gating backward on W consecutive elements: dA = dH*keep/(1-p); dU = dA*act(G); dG = dA*U*act'(G)
+template <typename T, int W, int ACT = ACT_RUNTIME>
+__device__ __forceinline__ void gating_bwd_core(int act, const DropoutParams& drop, size_t e, float* dh,
                                                 typename PackW<T, W>::type gp,
                                                 typename PackW<T, W>::type up, T* dg, T* du) {
   float dgv[W], duv[W];
@@ -365,21 +372,23 @@ __device__ __forceinline__ void gating_bwd_core(const DropoutParams& drop, size_
 #pragma unroll
     for (int r = 0; r < W; ++r) dh[r] = keep[r] ? dh[r] * drop.scale : 0.f;
   }
+  float gv[W], av[W], dv[W];
+#pragma unroll
+  for (int r = 0; r < W; ++r) gv[r] = Traits<T>::to_f32(gp[r]);
+  act_fwd_grad_w<W, ACT>(act, gv, av, dv);
 #pragma unroll
   for (int r = 0; r < W; ++r) {
-    float gv = Traits<T>::to_f32(gp[r]), uv = Traits<T>::to_f32(up[r]);
-    float s = sigmoid_f32(gv);
-    duv[r] = dh[r] * (gv * s);
-    dgv[r] = dh[r] * uv * (s * (1.0f + gv * (1.0f - s)));
+    duv[r] = dh[r] * av[r];
+    dgv[r] = dh[r] * Traits<T>::to_f32(up[r]) * dv[r];
   }
   store_w<T, W>(dg + e, dgv);
   store_w<T, W>(du + e, duv);
 }
 template <typename T, int W>
-__device__ __forceinline__ void gating_bwd_w(const DropoutParams& drop, size_t e, float* dh,
-                                             const T* g, const T* u, T* dg, T* du) {
+__device__ __forceinline__ void gating_bwd_w(int act, const DropoutParams& drop, size_t e,
+                                             float* dh, const T* g, const T* u, T* dg, T* du) {
   typedef typename PackW<T, W>::type pack;
-  gating_bwd_core<T, W>(drop, e, dh, *(const pack*)(g + e), *(const pack*)(u + e), dg, du);
+  gating_bwd_core<T, W>(act, drop, e, dh, *(const pack*)(g + e), *(const pack*)(u + e), dg, du);
 }
 
 template <typename T>
@@ -390,11 +399,12 @@ struct EpiDh {
     T* dg;
     T* du;
     int ldc;
+    int act;  // Act code
     DropoutParams drop;
   };
   template <int W>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*) {
-    gating_bwd_w<T, W>(a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
+    gating_bwd_w<T, W>(a.act, a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
   }
   // G and U come from HBM and every workgroup of a round reaches its epilogue at about the same
   // time; a kernel that can, fetches them this many W-wide items ahead of their use.
@@ -410,10 +420,11 @@ struct EpiDh {
     p.g = *(const pack*)(a.g + e);
     p.u = *(const pack*)(a.u + e);
   }
-  template <int W>
+  static constexpr bool HAS_ACT = true;
+  template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*,
                                                const Prefetch<W>& p) {
-    gating_bwd_core<T, W>(a.drop, (size_t)m * a.ldc + n, dh, p.g, p.u, a.dg, a.du);
+    gating_bwd_core<T, W, ACT>(a.act, a.drop, (size_t)m * a.ldc + n, dh, p.g, p.u, a.dg, a.du);
   }
 };
 

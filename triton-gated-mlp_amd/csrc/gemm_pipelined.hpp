@@ -303,45 +303,53 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   float* stg = (float*)(smem + wave * Cfg::EPI_WAVE_BYTES);
   const int mrow = lane & (MI - 1), nsub = 4 * (lane / MI);
   constexpr int NV = MI == 32 ? 4 : 1;  // 4-column vectors a lane holds per accumulator
+  // The slab loop exists once per activation choice the epilogue offers (SiLU fixed at compile
+  // time, or read at run time): a run-time switch inside it would leave the usual path threading
+  // its way through several times its own code.
+  auto slabs = [&](auto act_c) __attribute__((always_inline)) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const int b = g / TN, j = g % TN;
+      for (int g = 0; g < G; ++g) {
+        const int b = g / TN, j = g % TN;
 #pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        f32x4 o;
+        for (int v = 0; v < NV; ++v) {
+          f32x4 o;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = acc[g][i][4 * v + r];
-        *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
+          for (int r = 0; r < 4; ++r) o[r] = acc[g][i][4 * v + r];
+          *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
+        }
       }
-    }
-    // Same-wavefront LDS writes and reads are ordered; no barrier needed for a private slab.
+      // Same-wavefront LDS writes and reads are ordered; no barrier needed for a private slab.
 #pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      const int q = i * ITEMS + it;
-      int row, m, n, cg;
-      item_pos(q, row, m, n, cg);
-      alignas(16) float v0[8], v1[8];
-      const float* p0 = stg + row * ELD + cg * 8;
-      *(f32x4*)v0 = *(const f32x4*)p0;
-      *(f32x4*)(v0 + 4) = *(const f32x4*)(p0 + 4);
-      if (NB == 2) {
-        const float* p1 = p0 + MI * ELD;
-        *(f32x4*)v1 = *(const f32x4*)p1;
-        *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
-      }
-      if (PD > 0) {
-        Epi::template apply<8>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
+      for (int it = 0; it < ITEMS; ++it) {
+        const int q = i * ITEMS + it;
+        int row, m, n, cg;
+        item_pos(q, row, m, n, cg);
+        alignas(16) float v0[8], v1[8];
+        const float* p0 = stg + row * ELD + cg * 8;
+        *(f32x4*)v0 = *(const f32x4*)p0;
+        *(f32x4*)(v0 + 4) = *(const f32x4*)(p0 + 4);
+        if (NB == 2) {
+          const float* p1 = p0 + MI * ELD;
+          *(f32x4*)v1 = *(const f32x4*)p1;
+          *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
+        }
+        Epi::template apply<8, ACT>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
         if (q + PD < NITEMS) {
           int row2, m2, n2, cg2;
           item_pos(q + PD, row2, m2, n2, cg2);
           Epi::template prefetch<8>(ea, m2, n2, pf[q % (PD > 0 ? PD : 1)]);
         }
-      } else {
-        Epi::template apply<8>(ea, m, n, v0, v1);
       }
     }
+  };
+  if constexpr (Epi::HAS_ACT) {
+    if (ea.act == ACT_SILU) slabs(std::integral_constant<int, ACT_SILU>{});
+    else slabs(std::integral_constant<int, ACT_RUNTIME>{});
+  } else {
+    slabs(std::integral_constant<int, ACT_RUNTIME>{});
   }
 }
 

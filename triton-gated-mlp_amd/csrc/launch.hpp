@@ -49,19 +49,20 @@ hipError_t launch_gemm(const GemmArgs& ga, const typename Epi::Args& ea, hipStre
 // decode.hip
 template <typename T>
 hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
-                         const T* bu, const T* bd, T* h, T* y, int M, int K, int N, hipStream_t s);
+                         const T* bu, const T* bd, T* h, T* y, int M, int K, int N, int act,
+                         hipStream_t s);
 
 // decode_stream.hip: LDS-ring streaming variant for K % 256 == 0 and N % 256 == 0
 bool decode_stream_supported(int M, int K, int N);
 template <typename T>
 hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
                                 const T* bu, const T* bd, T* h, T* y, int M, int K, int N,
-                                hipStream_t s);
+                                int act, hipStream_t s);
 
 // aux.hip
 template <typename T>
 hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
-                             const DropoutParams& d, hipStream_t s);
+                             int act, const DropoutParams& d, hipStream_t s);
 template <typename T>
 hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s);
 size_t colsum_workspace_bytes(int64_t M, int64_t C);

@@ -16,7 +16,20 @@ from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
+
+# hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
+# tables (src/triton_gated_mlp/gated_mlp.py:17-37).
+ACT_CODES = {
+    "silu": 0,
+    "swish": 0,
+    "gelu": 1,
+    "relu": 2,
+    "leaky_relu": 3,
+    "sigmoid": 4,
+    "tanh": 5,
+    "no_act": 6,
+}
 
 _STATUS_EXC = {-1: ValueError, -2: NotImplementedError, -3: ValueError, -4: RuntimeError}
 
@@ -30,15 +43,15 @@ _SIGNATURES = {
     "gmlp_abi_version": (_int, []),
     "gmlp_last_error": (ctypes.c_char_p, []),
     "gmlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
-    "gmlp_gateup_fwd": (_int, [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_gateup_fwd": (_int, [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
     "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr]),
-    "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
-    "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
     "gmlp_dx_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _i64, _int, _c_ptr]),
     "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr]),
     "gmlp_dw_bwd_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _c_ptr, _int, _c_ptr]),
     "gmlp_colsum": (_int, [_c_ptr] * 3 + [_i64, _i64, _int, _c_ptr]),
-    "gmlp_decode_fwd": (_int, [_c_ptr] * 10 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_decode_fwd": (_int, [_c_ptr] * 10 + [_i64, _i64, _i64, _int, _int, _c_ptr]),
     "gmlp_dropout_mask": (_int, [_c_ptr, _i64, _i64, _f32, _u64, _u64, _c_ptr]),
 }
 
@@ -91,6 +104,15 @@ def dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return GMLP_F32
     raise TypeError(f"fused gated-MLP kernels take float16, bfloat16 or float32 tensors, got {dtype}")
+
+
+def act_code(act_fn: str) -> int:
+    try:
+        return ACT_CODES[act_fn]
+    except KeyError:
+        raise NotImplementedError(
+            f"hidden_act {act_fn!r} is not one of {sorted(ACT_CODES)}"
+        ) from None
 
 
 def require_gpu(*tensors: Optional[Tensor]) -> torch.device:

@@ -8,8 +8,9 @@
 Reference: src/triton_gated_mlp/gated_mlp.py (EagerGatedMLP :73-98, eager_fwd/bwd :105-156,
 FusedGatedMLPFunction :159-200, FusedGatedMLP :203-237).  Differences, all towards the eager
 semantics: the fused path applies the gate/up/down biases and dropout (the reference drops them),
-returns bias gradients, keeps G and U from the forward pass instead of recomputing them, and runs
-the down projection and its backward in the same kernels family (one autograd node for the MLP).
+returns bias gradients, keeps G and U from the forward pass instead of recomputing them, runs the
+down projection and its backward in the same kernels family (one autograd node for the MLP), and
+implements every hidden_act of ACT_FWD (the reference's fused kernels know silu and no_act only).
 """
 
 from __future__ import annotations
@@ -94,17 +95,23 @@ def eager_bwd(x: Tensor, W_up: Tensor, W_gp: Tensor, grad_output: Tensor):
 
 
 class FusedGatedMLPFunction(Function):
-    """Hidden-state operator hidden = dropout(silu(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)).
+    """Hidden-state operator hidden = dropout(act_fn(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)).
 
-    Argument order (x, W_up, b_up, W_gp, b_gp) as in the reference; dropout_p/seed/offset are optional.
+    Argument order (x, W_up, b_up, W_gp, b_gp) as in the reference; dropout_p, seed, offset and
+    act_fn (default "silu") are optional.
     """
 
     @staticmethod
-    def forward(ctx, x, W_up, b_up, W_gp, b_gp, dropout_p: float = 0.0, seed: int = 0, offset: int = 0):
+    def forward(
+        ctx, x, W_up, b_up, W_gp, b_gp, dropout_p: float = 0.0, seed: int = 0, offset: int = 0, act_fn: str = "silu"
+    ):
         needs_grad = any(ctx.needs_input_grad[:5])
-        out = _fwd.gateup_fwd(x, W_gp, b_gp, W_up, b_up, dropout_p, seed, offset, save_activations=needs_grad)
+        out = _fwd.gateup_fwd(
+            x, W_gp, b_gp, W_up, b_up, dropout_p, seed, offset, save_activations=needs_grad, act_fn=act_fn
+        )
         if needs_grad:
             ctx.save_for_backward(x, W_up, W_gp, out.gate, out.up)
+        ctx.act_fn = act_fn
         ctx.dropout = (float(dropout_p), int(seed), int(offset))
         ctx.has_bias = (b_up is not None, b_gp is not None)
         return out.hidden
@@ -114,13 +121,13 @@ class FusedGatedMLPFunction(Function):
         x, W_up, W_gp, gate, up = ctx.saved_tensors
         p, seed, offset = ctx.dropout
         need = ctx.needs_input_grad
-        dg, du = _bwd.gating_bwd(grad_output, gate, up, p, seed, offset)
+        dg, du = _bwd.gating_bwd(grad_output, gate, up, p, seed, offset, ctx.act_fn)
         dx = _bwd.dx_bwd(dg, du, W_gp, W_up) if need[0] else None
         dW_up = _bwd.dw_bwd(du, x) if need[1] else None
         db_up = _bwd.colsum(du) if ctx.has_bias[0] and need[2] else None
         dW_gp = _bwd.dw_bwd(dg, x) if need[3] else None
         db_gp = _bwd.colsum(dg) if ctx.has_bias[1] and need[4] else None
-        grads = (dx, dW_up, db_up, dW_gp, db_gp, None, None, None)
+        grads = (dx, dW_up, db_up, dW_gp, db_gp, None, None, None, None)
         return grads[: len(need)]  # apply() may have been called with the 5 reference arguments only
 
 
@@ -128,10 +135,14 @@ class FusedGatedMLPFullFunction(Function):
     """Whole MLP as one autograd node, so dY -> (dG, dU) is a single GEMM with a fused epilogue."""
 
     @staticmethod
-    def forward(ctx, x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset, recompute=False):
+    def forward(
+        ctx, x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset, recompute=False, act_fn="silu"
+    ):
         needs_grad = any(ctx.needs_input_grad[:7])
         keep = needs_grad and not recompute
-        hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=keep)
+        hs = _fwd.gateup_fwd(
+            x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=keep, act_fn=act_fn
+        )
         y = _fwd.linear_fwd(hs.hidden, W_down, b_down)
         if keep:
             ctx.save_for_backward(x, W_gate, W_up, W_down, hs.gate, hs.up, hs.hidden)
@@ -140,6 +151,7 @@ class FusedGatedMLPFullFunction(Function):
             # run the gate/up GEMM again in backward; the dropout mask is a function of the seed
             ctx.save_for_backward(x, W_gate, W_up, W_down, b_gate, b_up)
         ctx.recompute = bool(recompute)
+        ctx.act_fn = act_fn
         ctx.dropout = (float(dropout_p), int(seed), int(offset))
         ctx.has_bias = (b_gate is not None, b_up is not None, b_down is not None)
         return y
@@ -149,7 +161,9 @@ class FusedGatedMLPFullFunction(Function):
         p, seed, offset = ctx.dropout
         if ctx.recompute:
             x, W_gate, W_up, W_down, b_gate, b_up = ctx.saved_tensors
-            hs = _fwd.gateup_fwd(x, W_gate, b_gate, W_up, b_up, p, seed, offset, save_activations=True)
+            hs = _fwd.gateup_fwd(
+                x, W_gate, b_gate, W_up, b_up, p, seed, offset, save_activations=True, act_fn=ctx.act_fn
+            )
             gate, up, hidden = hs.gate, hs.up, hs.hidden
         else:
             x, W_gate, W_up, W_down, gate, up, hidden = ctx.saved_tensors
@@ -158,7 +172,7 @@ class FusedGatedMLPFullFunction(Function):
         dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
         dw_jobs = []  # (slot, lhs, rhs): the weight gradients go out as one grouped launch
         if any(need[:5]):
-            dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset)
+            dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset, ctx.act_fn)
             if need[0]:
                 dx = _bwd.dx_bwd(dg, du, W_gate, W_up)
             if need[1]:
@@ -176,12 +190,12 @@ class FusedGatedMLPFullFunction(Function):
             dW_gate, dW_up, dW_down = grads.get("gate"), grads.get("up"), grads.get("down")
         if ctx.has_bias[2] and need[6]:
             db_down = _bwd.colsum(dy)
-        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None, None
+        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None, None, None
 
 
 class FusedGatedMLP(_GatedMLPBase):
     """Drop-in gated MLP running on hand-written gfx950 kernels (float16 / bfloat16 tuned; float32
-    on a compatibility path).
+    on a compatibility path).  `hidden_act` is any key of ACT_FWD.
 
     Dropout is active in training mode only.  The keep mask comes from a counter-based generator:
     set `dropout_seed` (int) for a fixed mask stream, otherwise each forward draws a seed from
@@ -194,10 +208,6 @@ class FusedGatedMLP(_GatedMLPBase):
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
-        if self.act_fn not in ("silu", "swish"):
-            raise NotImplementedError(
-                f"FusedGatedMLP implements hidden_act='silu' only, got {self.act_fn!r}; use EagerGatedMLP"
-            )
         self.dropout_seed: Optional[int] = None
         self.recompute_activations = False
         self._dropout_calls = 0
@@ -222,11 +232,13 @@ class FusedGatedMLP(_GatedMLPBase):
             x2.requires_grad or any(q.requires_grad for q in self.parameters())
         )
         if inference and p == 0.0 and _fwd.decode_supported(M, K, self.intermediate_size, x2.dtype):
-            y = _fwd.decode_fwd(x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias)
+            y = _fwd.decode_fwd(
+                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, self.act_fn
+            )
         else:
             seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
             y = FusedGatedMLPFullFunction.apply(
                 x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p, seed, offset,
-                self.recompute_activations,
+                self.recompute_activations, self.act_fn,
             )
         return y.reshape(*lead, self.hidden_size)

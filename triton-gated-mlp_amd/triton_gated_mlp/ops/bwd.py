@@ -18,7 +18,14 @@ from .fwd import _c, gateup_fwd
 
 
 def dh_bwd(
-    dy: Tensor, W_down: Tensor, g: Tensor, u: Tensor, dropout_p: float = 0.0, seed: int = 0, offset: int = 0
+    dy: Tensor,
+    W_down: Tensor,
+    g: Tensor,
+    u: Tensor,
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    act_fn: str = "silu",
 ) -> Tuple[Tensor, Tensor]:
     """(dG, dU) from dY: dH = dY·W_down with dropout and gating backward fused in the epilogue."""
     M, K = dy.shape
@@ -27,6 +34,7 @@ def dh_bwd(
         raise ValueError("dimension mismatch among dy, W_down, g, u")
     dev = _cabi.require_gpu(dy, W_down, g, u)
     code = _cabi.dtype_code(dy.dtype)
+    act = _cabi.act_code(act_fn)
     dy, W_down, g, u = _c(dy), _c(W_down), _c(g), _c(u)
     dg = torch.empty_like(g)
     du = torch.empty_like(u)
@@ -35,20 +43,27 @@ def dh_bwd(
             _cabi.check(
                 _cabi.lib().gmlp_dh_bwd(
                     _cabi.ptr(dy), _cabi.ptr(W_down), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du),
-                    M, K, N, code, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                    M, K, N, code, act, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
                 )
             )
     return dg, du
 
 
 def gating_bwd(
-    dh: Tensor, g: Tensor, u: Tensor, dropout_p: float = 0.0, seed: int = 0, offset: int = 0
+    dh: Tensor,
+    g: Tensor,
+    u: Tensor,
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    act_fn: str = "silu",
 ) -> Tuple[Tensor, Tensor]:
-    """(dG, dU) from dH (element-wise): dU = dA*silu(G), dG = dA*U*silu'(G), dA = dH*keep/(1-p)."""
+    """(dG, dU) from dH (element-wise): dU = dA*act(G), dG = dA*U*act'(G), dA = dH*keep/(1-p)."""
     if g.shape != dh.shape or u.shape != dh.shape or dh.ndim != 2:
         raise ValueError("dh, g, u must be 2-D tensors of one shape")
     dev = _cabi.require_gpu(dh, g, u)
     code = _cabi.dtype_code(dh.dtype)
+    act = _cabi.act_code(act_fn)
     dh, g, u = _c(dh), _c(g), _c(u)
     M, N = dh.shape
     dg = torch.empty_like(g)
@@ -57,7 +72,7 @@ def gating_bwd(
         with torch.cuda.device(dev):
             _cabi.check(
                 _cabi.lib().gmlp_gating_bwd(
-                    _cabi.ptr(dh), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du), M, N, code,
+                    _cabi.ptr(dh), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du), M, N, code, act,
                     float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
                 )
             )
@@ -175,15 +190,16 @@ def mlp_hidden_states_bwd(
     seed: int = 0,
     offset: int = 0,
     return_bias_grads: bool = False,
+    act_fn: str = "silu",
 ):
-    """Gradients of hidden = dropout(silu(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)) w.r.t. x, W_up, W_gp.
+    """Gradients of hidden = dropout(act_fn(x·W_gpᵀ+b_gp) * (x·W_upᵀ+b_up)) w.r.t. x, W_up, W_gp.
 
     Returns (dx, dW_up, dW_gp), or (dx, dW_up, db_up, dW_gp, db_gp) with return_bias_grads.
     """
     if gate is None or up is None:
-        fwd = gateup_fwd(x, W_gp, b_gp, W_up, b_up, 0.0, 0, 0, save_activations=True)
+        fwd = gateup_fwd(x, W_gp, b_gp, W_up, b_up, 0.0, 0, 0, save_activations=True, act_fn=act_fn)
         gate, up = fwd.gate, fwd.up
-    dg, du = gating_bwd(grad_output, gate, up, dropout_p, seed, offset)
+    dg, du = gating_bwd(grad_output, gate, up, dropout_p, seed, offset, act_fn)
     dx = dx_bwd(dg, du, W_gp, W_up)
     dW_up = dw_bwd(du, x)
     dW_gp = dw_bwd(dg, x)

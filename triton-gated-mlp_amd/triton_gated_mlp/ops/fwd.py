@@ -54,9 +54,11 @@ def gateup_fwd(
     offset: int = 0,
     save_activations: bool = False,
     return_mask: bool = False,
+    act_fn: str = "silu",
 ) -> HiddenStates:
-    """H = dropout(silu(x·W_gateᵀ + b_gate) * (x·W_upᵀ + b_up)) in one kernel."""
+    """H = dropout(act_fn(x·W_gateᵀ + b_gate) * (x·W_upᵀ + b_up)) in one kernel."""
     validate_dimensions(x, W_up, b_up, W_gate, b_gate)
+    act = _cabi.act_code(act_fn)
     dev = _cabi.require_gpu(x, W_gate, b_gate, W_up, b_up)
     code = _cabi.dtype_code(x.dtype)
     x, W_gate, W_up, b_gate, b_up = _c(x), _c(W_gate), _c(W_up), _c(b_gate), _c(b_up)
@@ -72,7 +74,7 @@ def gateup_fwd(
                 _cabi.lib().gmlp_gateup_fwd(
                     _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(b_gate), _cabi.ptr(b_up),
                     _cabi.ptr(h), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(mask),
-                    M, K, N, code, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                    M, K, N, code, act, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
                 )
             )
     return HiddenStates(h, g, u, mask)
@@ -90,10 +92,13 @@ def mlp_hidden_states_fwd(
     seed: int = 0,
     offset: int = 0,
 ) -> Tensor:
-    """dropout(act_fn(gate_proj(x)) * up_proj(x)) fused; weights in nn.Linear [N, K] layout."""
-    if act_fn not in ("silu", "swish"):
-        raise NotImplementedError(f"fused gated MLP supports act_fn='silu' only, got {act_fn!r}")
-    return gateup_fwd(x, WT_gp, b_gp, WT_up, b_up, dropout_p, seed, offset).hidden
+    """dropout(act_fn(gate_proj(x)) * up_proj(x)) fused; weights in nn.Linear [N, K] layout.
+
+    act_fn is any name of the reference's activation table (silu, swish, gelu, relu, leaky_relu,
+    sigmoid, tanh, no_act); an unknown name raises NotImplementedError like the reference's
+    _act_fwd (src/triton_gated_mlp/ops/act.py:5-12).
+    """
+    return gateup_fwd(x, WT_gp, b_gp, WT_up, b_up, dropout_p, seed, offset, act_fn=act_fn).hidden
 
 
 def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
@@ -134,6 +139,7 @@ def decode_fwd(
     b_up: Optional[Tensor],
     W_down: Tensor,
     b_down: Optional[Tensor],
+    act_fn: str = "silu",
 ) -> Tensor:
     """Whole-MLP forward for M <= 16 token rows: every weight byte is read from HBM once."""
     validate_dimensions(x, W_up, b_up, W_gate, b_gate)
@@ -143,6 +149,7 @@ def decode_fwd(
         raise ValueError(f"dimension mismatch in W_down {tuple(W_down.shape)}")
     dev = _cabi.require_gpu(x, W_gate, b_gate, W_up, b_up, W_down, b_down)
     code = _cabi.dtype_code(x.dtype)
+    act = _cabi.act_code(act_fn)
     x, W_gate, W_up, W_down = _c(x), _c(W_gate), _c(W_up), _c(W_down)
     b_gate, b_up, b_down = _c(b_gate), _c(b_up), _c(b_down)
     h = torch.empty((M, N), dtype=x.dtype, device=dev)
@@ -151,7 +158,7 @@ def decode_fwd(
         _cabi.check(
             _cabi.lib().gmlp_decode_fwd(
                 _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(W_down), _cabi.ptr(b_gate),
-                _cabi.ptr(b_up), _cabi.ptr(b_down), _cabi.ptr(h), _cabi.ptr(y), None, M, K, N, code,
+                _cabi.ptr(b_up), _cabi.ptr(b_down), _cabi.ptr(h), _cabi.ptr(y), None, M, K, N, code, act,
                 _cabi.stream_ptr(dev),
             )
         )
