@@ -89,8 +89,10 @@ int hip_result(const char* fn, hipError_t e) {
 // LARGE tiles need whole 256 x bn_large tiles, a reduction that is a multiple of 64, and enough
 // tiles to occupy the chip; whole 128 x (bn_large/2) tiles run on MEDIUM_FULL; everything else on
 // the predicated MEDIUM class.  The pipelined kernels address operands with 32-bit byte offsets.
-int pick_tile(int64_t rows, int64_t cols, int64_t red, int bn_large) {
-  const int64_t limit = (int64_t)1 << 31;
+int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large) {
+  if (dtype == GMLP_F32) return gmlp::TILE_MEDIUM;  // the float32 kernel has one tile shape
+  // 32-bit buffer offsets from a base that sits up to 4 KB below the operand (shared-M0 loads)
+  const int64_t limit = ((int64_t)1 << 31) - 4096;
   bool offsets_fit = rows * red * 2 < limit && cols * red * 2 < limit;
   if (!offsets_fit || red % 64 != 0) return gmlp::TILE_MEDIUM;
   if (rows % 256 == 0 && cols % bn_large == 0 && (rows / 256) * (cols / bn_large) >= 192)
@@ -134,7 +136,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   ga.A[0] = x; ga.A[1] = x; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
   ga.nseg = 1; ga.group_m = 8;
-  int tc = pick_tile(M, N, K, 128);
+  int tc = pick_tile(dtype, M, N, K, 128);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -160,7 +162,7 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   ga.A[0] = a; ga.A[1] = a; ga.B[0] = w; ga.B[1] = w;
   ga.M = (int)M; ga.N = (int)C; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
   ga.nseg = 1; ga.group_m = 8;
-  int tc = pick_tile(M, C, R, 256);
+  int tc = pick_tile(dtype, M, C, R, 256);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -191,7 +193,7 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   ga.A[0] = dy; ga.A[1] = dy; ga.B[0] = w_down; ga.B[1] = w_down;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
   ga.nseg = 1; ga.group_m = 8;
-  int tc = pick_tile(M, N, K, 256);
+  int tc = pick_tile(dtype, M, N, K, 256);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -240,7 +242,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   ga.A[0] = dg; ga.A[1] = du; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
   ga.nseg = 2; ga.group_m = 8;
-  int tc = pick_tile(M, K, N, 256);
+  int tc = pick_tile(dtype, M, K, N, 256);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -265,7 +267,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   ga.A[0] = lhs; ga.A[1] = lhs; ga.B[0] = rhs; ga.B[1] = rhs;
   ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
   ga.nseg = 1; ga.group_m = 8;
-  int tc = pick_tile(R, C, Mred, 256);
+  int tc = pick_tile(dtype, R, C, Mred, 256);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -290,7 +292,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     if (int rc = check_mult8(__func__, "R", R[i])) return rc;
     if (int rc = check_mult8(__func__, "C", C[i])) return rc;
     GMLP_REQUIRE_ALIGNED(lhs[i]); GMLP_REQUIRE_ALIGNED(rhs[i]); GMLP_REQUIRE_ALIGNED(dw[i]);
-    large = large && dtype != GMLP_F32 && pick_tile(R[i], C[i], Mred, 256) == TILE_LARGE;
+    large = large && pick_tile(dtype, R[i], C[i], Mred, 256) == TILE_LARGE;
   }
   if (!large) {
     for (int i = 0; i < count; ++i)
@@ -304,24 +306,20 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     ga.M = (int)R[i]; ga.N = (int)C[i]; ga.K = (int)Mred; ga.lda = (int)R[i]; ga.ldb = (int)C[i];
     ga.nseg = 1; ga.group_m = 8;
   };
-  hipError_t e;
-  if (dtype == GMLP_F16) {
-    GemmGroup<EpiStore<f16>::Args> grp = {};
-    grp.count = count;
-    for (int i = 0; i < count; ++i) {
-      fill(grp.ga[i], i);
-      grp.ea[i] = EpiStore<f16>::Args{(f16*)dw[i], nullptr, (int)C[i]};
+  hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
+    typedef decltype(tag) T;
+    if constexpr (std::is_same<T, float>::value) {
+      return hipErrorInvalidValue;  // not reached: float32 problems take the separate launches above
+    } else {
+      GemmGroup<typename EpiStore<T>::Args> grp = {};
+      grp.count = count;
+      for (int i = 0; i < count; ++i) {
+        fill(grp.ga[i], i);
+        grp.ea[i] = typename EpiStore<T>::Args{(T*)dw[i], nullptr, (int)C[i]};
+      }
+      return launch_dw_group<T>(grp, s);
     }
-    e = launch_dw_group<f16>(grp, s);
-  } else {
-    GemmGroup<EpiStore<bf16>::Args> grp = {};
-    grp.count = count;
-    for (int i = 0; i < count; ++i) {
-      fill(grp.ga[i], i);
-      grp.ea[i] = EpiStore<bf16>::Args{(bf16*)dw[i], nullptr, (int)C[i]};
-    }
-    e = launch_dw_group<bf16>(grp, s);
-  }
+  });
   return hip_result(__func__, e);
 }
 

@@ -29,6 +29,9 @@ namespace gmlp {
 #ifndef GMLP_LOAD_CYCLES
 #define GMLP_LOAD_CYCLES 64  // one global->LDS load per this many MFMA cycles
 #endif
+#ifndef GMLP_B_LOOKAHEAD
+#define GMLP_B_LOOKAHEAD 2  // MFMA groups between the fetch of a B fragment and its use (2 or 3)
+#endif
 
 template <int MI>
 struct AccType;
@@ -83,7 +86,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   constexpr int KSTEPS = Cfg::KSTEPS, STAGE = Cfg::STAGE, L = Cfg::LOADS;
   constexpr int LOAD_SLOTS = GMLP_LOAD_CYCLES / Cfg::MFMA_CYCLES;  // MFMA slots per load
   constexpr int TILE_SLOTS = KSTEPS * G * TM;                         // MFMA slots per tile
-  constexpr int HEAD_SLOTS = 2 * TM;  // slots between the retiring barrier and the tile's end
+  constexpr int LA = GMLP_B_LOOKAHEAD;
+  static_assert(LA >= 2 && LA <= 3 && LA <= G, "B ring has 4 entries");
+  constexpr int HEAD_SLOTS = LA * TM;  // slots between the retiring barrier and the tile's end
   // Fragment fetches sit in slots 0 and 1 of a group; with four or more slots per load the loads
   // keep away from them.
   constexpr int LOAD_PHASE = LOAD_SLOTS >= 4 ? 2 : 0;
@@ -204,8 +209,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
       const bool last = ks == KSTEPS - 1;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const bool handover = last && g >= G - 2;  // groups that already work for tile kt+1
-        if (NEXT && last && g == G - 2) {
+        const bool handover = last && g >= G - LA;  // groups that already work for tile kt+1
+        if (NEXT && last && g == G - LA) {
           // No fetch addresses this tile's slot any more: wait until tile kt+1 has landed,
           // barrier, then the slot can be refilled.
           wait_vmem<0>();
@@ -216,9 +221,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           acc[g][i] = mfma_mi<T, MI>(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
-          // --- B fragment of the group two ahead
+          // --- B fragment of the group LA ahead
           if (i == 0) {
-            const int g2 = g + 2;
+            const int g2 = g + LA;
             if (g2 < G) fetch_b((ks * G + g2) % 4, g2, kt, ks);
             else if (!last) fetch_b(((ks + 1) * G + g2 - G) % 4, g2 - G, kt, ks + 1);
             else if (NEXT) fetch_b((g2 - G) % 4, g2 - G, kt + 1, 0);
@@ -227,14 +232,15 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           if (!last) {
             if (i == 1 && g < TM) fetch_a((ks + 1) & 1, g, kt, ks + 1);
           } else if (NEXT && handover) {
-            const int h = (g - (G - 2)) * (TM / 2) + (i - 1);
-            if (i >= 1 && i <= TM / 2) fetch_a(0, h, kt + 1, 0);
+            constexpr int AH = (TM + LA - 1) / LA;  // A fragments per handover group
+            const int h = (g - (G - LA)) * AH + (i - 1);
+            if (i >= 1 && i <= AH && h < TM) fetch_a(0, h, kt + 1, 0);
           }
           // --- paced refill of the ring slot retired at the last barrier; slots are counted from
           // that barrier, so a tile's loads start in the previous tile's handover groups.  Load x
           // goes to slot x*LOAD_SLOTS + LOAD_PHASE, a new M0 one slot earlier.
           if (NEXT) {
-            const int slot = handover ? (g - (G - 2)) * TM + i : HEAD_SLOTS + (ks * G + g) * TM + i;
+            const int slot = handover ? (g - (G - LA)) * TM + i : HEAD_SLOTS + (ks * G + g) * TM + i;
             const int lkt = handover ? kt + NS : kt + NS - 1;
             if (slot % LOAD_SLOTS == LOAD_PHASE && slot / LOAD_SLOTS < L)
               issue_one(lkt, slot / LOAD_SLOTS);
@@ -265,8 +271,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < TM; ++i) fetch_a(0, i, 0, 0);
-  fetch_b(0, 0, 0, 0);
-  fetch_b(1, 1, 0, 0);
+#pragma unroll
+  for (int g = 0; g < LA; ++g) fetch_b(g, g, 0, 0);
   __builtin_amdgcn_sched_barrier(0);
 
   // Epilogue work items of a wavefront: MI-row slab i of its tile, then (row, 8-column group)
