@@ -132,6 +132,22 @@ def test_small_shapes_forward_backward(M, K, N, bias, p, dtype):
     _run_module_case(Case(f"small_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=p, backward=True, seed=M + K + N))
 
 
+@pytest.mark.parametrize(
+    "M,K,N,dtype,bias,p",
+    [
+        (3001, 2048, 4096, torch.float16, False, 0.0),  # odd token count on the 256-tile and 128-tile kernels
+        (1000, 1024, 4104, torch.bfloat16, True, 0.1),  # ragged tokens and ragged intermediate size
+        (50, 512, 1024, torch.float16, True, 0.0),  # fewer rows than one tile
+        (4099, 1024, 2048, torch.float16, False, 0.0),  # three rows into the last tile-row
+    ],
+)
+def test_ragged_token_counts_on_the_pipelined_kernels(M, K, N, dtype, bias, p):
+    """Token counts (and intermediate sizes) that are not multiples of the tile run on the same
+    kernels as whole tiles: the part of a tile beyond the end of an operand reads as zero.  The
+    weight gradients reduce over the ragged dimension."""
+    _run_module_case(Case(f"ragged_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=p, backward=True, seed=M))
+
+
 OTHER_ACTS = ["gelu", "relu", "leaky_relu", "sigmoid", "tanh", "no_act"]
 
 

@@ -86,19 +86,25 @@ int hip_result(const char* fn, hipError_t e) {
   return fail(GMLP_EHIP, "%s: HIP error %d (%s)", fn, (int)e, hipGetErrorString(e));
 }
 
-// LARGE tiles need whole 256 x bn_large tiles, a reduction that is a multiple of 64, and enough
-// tiles to occupy the chip; whole 128 x (bn_large/2) tiles run on MEDIUM_FULL; everything else on
-// the predicated MEDIUM class.  The pipelined kernels address operands with 32-bit byte offsets.
-int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large) {
+// Tile class for an output of rows x cols with reduction length red (all in elements).
+// The pipelined kernels (LARGE: 256 x bn_large tiles, one workgroup per CU; MEDIUM_FULL: tiles of
+// half that in each direction, two per CU) take any rows and cols; they need 32-bit byte offsets
+// into the operands, padded to whole tiles, and a reduction that is a multiple of 64 unless both
+// operands are reduction-strided (`both_ks`).  Everything else runs on the predicated MEDIUM class.
+// Between the two pipelined classes the choice is padded work, with the small tiles counted at
+// the 75 % of the large tiles' throughput they reach, and enough large tiles to occupy the chip.
+int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large, bool both_ks = false) {
   if (dtype == GMLP_F32) return gmlp::TILE_MEDIUM;  // the float32 kernel has one tile shape
-  // 32-bit buffer offsets from a base that sits up to 4 KB below the operand (shared-M0 loads)
+  auto up = [](int64_t v, int64_t q) { return (v + q - 1) / q * q; };
+  // the buffer base sits up to 4 KB below the operand (shared-M0 loads)
   const int64_t limit = ((int64_t)1 << 31) - 4096;
-  bool offsets_fit = rows * red * 2 < limit && cols * red * 2 < limit;
-  if (!offsets_fit || red % 64 != 0) return gmlp::TILE_MEDIUM;
-  if (rows % 256 == 0 && cols % bn_large == 0 && (rows / 256) * (cols / bn_large) >= 192)
-    return gmlp::TILE_LARGE;
-  if (rows % 128 == 0 && cols % (bn_large / 2) == 0) return gmlp::TILE_MEDIUM_FULL;
-  return gmlp::TILE_MEDIUM;
+  bool offsets_fit = up(rows, 256) * up(red, 64) * 2 < limit && up(cols, 256) * up(red, 64) * 2 < limit;
+  if (!offsets_fit || (red % 64 != 0 && !both_ks)) return gmlp::TILE_MEDIUM;
+  const int64_t large_tiles = (up(rows, 256) / 256) * (up(cols, bn_large) / bn_large);
+  const double large_work = (double)up(rows, 256) * up(cols, bn_large);
+  const double medium_work = (double)up(rows, 128) * up(cols, bn_large / 2) / 0.75;
+  if (large_tiles >= 192 && large_work <= medium_work) return gmlp::TILE_LARGE;
+  return gmlp::TILE_MEDIUM_FULL;
 }
 
 }  // namespace
@@ -267,7 +273,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   ga.A[0] = lhs; ga.A[1] = lhs; ga.B[0] = rhs; ga.B[1] = rhs;
   ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
   ga.nseg = 1; ga.group_m = 8;
-  int tc = pick_tile(dtype, R, C, Mred, 256);
+  int tc = pick_tile(dtype, R, C, Mred, 256, true);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -292,7 +298,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     if (int rc = check_mult8(__func__, "R", R[i])) return rc;
     if (int rc = check_mult8(__func__, "C", C[i])) return rc;
     GMLP_REQUIRE_ALIGNED(lhs[i]); GMLP_REQUIRE_ALIGNED(rhs[i]); GMLP_REQUIRE_ALIGNED(dw[i]);
-    large = large && pick_tile(dtype, R[i], C[i], Mred, 256) == TILE_LARGE;
+    large = large && pick_tile(dtype, R[i], C[i], Mred, 256, true) == TILE_LARGE;
   }
   if (!large) {
     for (int i = 0; i < count; ++i)

@@ -1,11 +1,19 @@
 // Pipelined full-tile MFMA GEMM for gfx950.
 //
 // Same contract as gemm_kernel (gemm.hpp): C[M,N] = sum_s sum_k A_s[m,k] * B_s[n,k], operands
-// reduction-contiguous (KC) or reduction-strided (KS), NB accumulator sets, fused epilogue; but
-// restricted to whole BM x BN tiles and K % 64 == 0.  Reduction tiles of 64 elements travel
-// global -> LDS without passing through registers (gemm_tiles.hpp) into a two-slot ring; the
-// epilogue transposes accumulators through LDS so that every global access is a 16-byte,
-// row-contiguous one.
+// reduction-contiguous (KC) or reduction-strided (KS), NB accumulator sets, fused epilogue.
+// Reduction tiles of 64 elements travel global -> LDS without passing through registers
+// (gemm_tiles.hpp) into a two-slot ring; the epilogue transposes accumulators through LDS so that
+// every global access is a 16-byte, row-contiguous one.
+//
+// Ragged edges cost nothing in the main loop: operands are read through buffer descriptors of
+// their exact size, so whatever a tile addresses beyond the END of an operand reads as zero.
+//   * M and N need not be multiples of the tile: rows of a KC operand beyond the last one lie
+//     beyond its end; columns of a KS operand beyond the last one alias the next reduction row,
+//     which only feeds output rows/columns that the epilogue does not store.
+//   * K need not be a multiple of 64 when BOTH operands are KS (reduction rows beyond K lie beyond
+//     the end: the weight gradients, whose reduction runs over the tokens).  With a KC operand K
+//     must be a multiple of 64 (its tail would alias the next row); the host checks.
 //
 // Per 512/MI-wide reduction step a wavefront issues G groups of TM MFMAs: group g multiplies one
 // B fragment (accumulator set b, column block j; G = NB * TN) with the step's TM A fragments.
@@ -102,7 +110,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
-  const int tiles_m = ga.M / BM, tiles_n = ga.N / BN;
+  const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
   int tm_i, tn_i;
   map_tile(pid, nwg, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
   const int m0 = tm_i * BM, n0 = tn_i * BN;
@@ -115,7 +123,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 #pragma unroll
       for (int r = 0; r < (int)(sizeof(acc_t) / 4); ++r) acc[g][i][r] = 0.f;
 
-  const int kt_seg = ga.K / BK;
+  const int kt_seg = (ga.K + BK - 1) / BK;
   const int kt_total = kt_seg * ga.nseg;
 
   // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
@@ -136,10 +144,12 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const uint32_t a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
   const uint32_t b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem;
-  const buffer_rsrc ra[2] = {make_rsrc((const char*)ga.A[0] - DMA_BIAS),
-                             make_rsrc((const char*)ga.A[1] - DMA_BIAS)};
-  const buffer_rsrc rb[2] = {make_rsrc((const char*)ga.B[0] - DMA_BIAS),
-                             make_rsrc((const char*)ga.B[1] - DMA_BIAS)};
+  const uint32_t a_bytes = (uint32_t)(A_KS ? ga.K : ga.M) * ga.lda * 2 + DMA_BIAS;
+  const uint32_t b_bytes = (uint32_t)(B_KS ? ga.K : ga.N) * ga.ldb * 2 + DMA_BIAS;
+  const buffer_rsrc ra[2] = {make_rsrc((const char*)ga.A[0] - DMA_BIAS, a_bytes),
+                             make_rsrc((const char*)ga.A[1] - DMA_BIAS, a_bytes)};
+  const buffer_rsrc rb[2] = {make_rsrc((const char*)ga.B[0] - DMA_BIAS, b_bytes),
+                             make_rsrc((const char*)ga.B[1] - DMA_BIAS, b_bytes)};
 
   // Global->LDS load number x (0 .. L-1) of this wavefront for reduction tile kt_req: operand and
   // index within the operand's loads.
@@ -277,7 +287,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 
   // Epilogue work items of a wavefront: MI-row slab i of its tile, then (row, 8-column group)
   // items spread over the lanes.  What an epilogue reads from global memory is fetched
-  // PREFETCH_DEPTH items ahead, starting before the last reduction tile.
+  // PREFETCH_DEPTH items ahead, starting before the last reduction tile; items beyond the edge of
+  // the output fetch the last valid row / column group instead (no branch around the loads) and
+  // are dropped when it comes to storing.
   constexpr int ITEMS = MI * WTN / 8 / 64;  // items per lane and slab
   constexpr int NITEMS = TM * ITEMS;
   constexpr int PD = Epi::PREFETCH_DEPTH < NITEMS ? Epi::PREFETCH_DEPTH : NITEMS;
@@ -297,7 +309,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   for (int q = 0; q < PD; ++q) {
     int row, m, n, cg;
     item_pos(q, row, m, n, cg);
-    Epi::template prefetch<8>(ea, m, n, pf[q]);
+    Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
   }
   tile_body(kt, std::false_type{});
   wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
@@ -342,11 +354,11 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           *(f32x4*)v1 = *(const f32x4*)p1;
           *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
         }
-        Epi::template apply<8, ACT>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
+        if (m < ga.M && n < ga.N) Epi::template apply<8, ACT>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
         if (q + PD < NITEMS) {
           int row2, m2, n2, cg2;
           item_pos(q + PD, row2, m2, n2, cg2);
-          Epi::template prefetch<8>(ea, m2, n2, pf[q % (PD > 0 ? PD : 1)]);
+          Epi::template prefetch<8>(ea, min(m2, ga.M - 1), min(n2, ga.N - 8), pf[q % (PD > 0 ? PD : 1)]);
         }
       }
     }
@@ -389,7 +401,7 @@ hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& e
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
-  dim3 grid((ga.M / BM) * (ga.N / BN)), block(Cfg::NW * 64);
+  dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN)), block(Cfg::NW * 64);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
   return hipGetLastError();
 }
@@ -403,7 +415,7 @@ hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipSt
   int total = 0;
   for (int g = 0; g < grp.count; ++g) {
     grp.first[g] = total;
-    total += (grp.ga[g].M / BM) * (grp.ga[g].N / BN);
+    total += ((grp.ga[g].M + BM - 1) / BM) * ((grp.ga[g].N + BN - 1) / BN);
   }
   for (int g = grp.count; g <= GEMM_GROUP_MAX; ++g) grp.first[g] = total;
   hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);

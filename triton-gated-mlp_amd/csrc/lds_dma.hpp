@@ -10,10 +10,12 @@ typedef short i16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef int buffer_rsrc __attribute__((ext_vector_type(4)));
 
-// Raw buffer descriptor over the whole address range behind `base` (offsets are 32-bit bytes).
-__device__ __forceinline__ buffer_rsrc make_rsrc(const void* base) {
+// Raw buffer descriptor over `bytes` bytes behind `base` (offsets are 32-bit bytes).  The hardware
+// range-checks voffset + soffset + immediate offset against `bytes`, per dword: what lies beyond
+// reads as zero, also into LDS, and never faults (checked on gfx950 with a stand-alone probe).
+__device__ __forceinline__ buffer_rsrc make_rsrc(const void* base, uint32_t bytes = 0x7FFFFFFFu) {
   uint64_t b = (uint64_t)base;
-  buffer_rsrc r = {(int)(uint32_t)b, (int)((b >> 32) & 0xffffu), 0x7FFFFFFF, 0x00020000};
+  buffer_rsrc r = {(int)(uint32_t)b, (int)((b >> 32) & 0xffffu), (int)bytes, 0x00020000};
   return r;
 }
 // 16 bytes per lane from (rsrc base + soffset + voffset) to LDS byte address (lds_wave_base +
