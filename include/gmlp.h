@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 2
+#define GMLP_ABI_VERSION 3
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -61,12 +61,16 @@ enum gmlp_status {
   GMLP_EHIP = -4    /* HIP runtime reported an error at launch */
 };
 
-enum gmlp_op { GMLP_OP_DECODE_FWD = 0, GMLP_OP_COLSUM = 1 };
+enum gmlp_op { GMLP_OP_DECODE_FWD = 0, GMLP_OP_COLSUM = 1, GMLP_OP_LINEAR_FWD = 2, GMLP_OP_DX_BWD = 3 };
 
 int gmlp_abi_version(void);
 const char* gmlp_last_error(void);
 
-/* Workspace bytes the caller must provide for `op` at the given problem size (0 if none). */
+/*
+ * Workspace bytes the caller must provide for `op` at the given problem size (0 if none), with
+ * (M, K, N) as the entry point of that name takes them: GMLP_OP_COLSUM (M, 0, C),
+ * GMLP_OP_LINEAR_FWD (M, R, C), GMLP_OP_DX_BWD (M, K, N), GMLP_OP_DECODE_FWD (M, K, N).
+ */
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
 
 /*
@@ -87,9 +91,13 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
  * Linear layer forward: out[M,C] = a[M,R]·w[C,R]ᵀ + bias[C]   (bias may be NULL).
  * Replaces the nn.Linear down_proj call (src/triton_gated_mlp/gated_mlp.py:236), which the
  * reference leaves to the vendor BLAS.  Requires R % 8 == 0, C % 8 == 0.
+ * workspace (may be NULL): gmlp_workspace_bytes(GMLP_OP_LINEAR_FWD, M, R, C, dtype) bytes.  It is
+ * non-zero for outputs of a few tiles with a long reduction (short batches): with it the reduction
+ * is split over several workgroups per tile (fp32 partial sums, added in a fixed order); without
+ * it the same result comes from one workgroup per tile, several times slower on such shapes.
  */
 int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, int64_t M, int64_t R,
-                    int64_t C, int dtype, void* stream);
+                    int64_t C, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Backward through down_proj, dropout and the gating product in one GEMM:
@@ -114,9 +122,12 @@ int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void
 /*
  * dX = dG·W_gate + dU·W_up   (one GEMM over the concatenated reduction of length 2N).
  * Replaces _compute_dx (src/triton_gated_mlp/ops/bwd.py:242-322; gated_mlp.py:147-149).
+ * workspace (may be NULL): gmlp_workspace_bytes(GMLP_OP_DX_BWD, M, K, N, dtype) bytes, used as in
+ * gmlp_linear_fwd.
  */
 int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* w_up, void* dx,
-                int64_t M, int64_t K, int64_t N, int dtype, void* stream);
+                int64_t M, int64_t K, int64_t N, int dtype, void* workspace, size_t workspace_bytes,
+                void* stream);
 
 /*
  * Weight gradient: dw[R,C] = lhs[Mred,R]ᵀ · rhs[Mred,C].

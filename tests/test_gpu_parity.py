@@ -148,6 +148,46 @@ def test_ragged_token_counts_on_the_pipelined_kernels(M, K, N, dtype, bias, p):
     _run_module_case(Case(f"ragged_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=p, backward=True, seed=M))
 
 
+@pytest.mark.parametrize(
+    "M,K,N,dtype,bias",
+    [
+        (17, 2048, 8192, torch.float16, True),  # one more row than the skinny-M kernels take
+        (64, 1024, 4096, torch.float16, False),
+        (300, 1024, 4096, torch.bfloat16, True),
+        (130, 4096, 14336, torch.float16, False),  # Llama-3-8B widths, short batch
+    ],
+)
+def test_short_batches_split_the_long_reductions(M, K, N, dtype, bias):
+    """Down projection and input gradient of a short batch have a few output tiles and a long
+    reduction; the library asks for a workspace and splits the reduction over several workgroups
+    per tile.  Same results as ever, to the usual tolerance."""
+    from triton_gated_mlp import _cabi
+
+    code = _cabi.dtype_code(dtype)
+    assert _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, M, N, K, code) > 0
+    assert _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_DX_BWD, M, K, N, code) > 0
+    _run_module_case(Case(f"short_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=0.0, backward=True, seed=M + 1))
+
+
+def test_split_reduction_without_workspace_gives_the_unsplit_result():
+    """NULL workspace is always accepted: one workgroup per tile, same numbers up to summation order."""
+    from triton_gated_mlp import _cabi
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(48, 8192, generator=g).to(torch.float16).to(dev)
+    W = (0.02 * torch.randn(1024, 8192, generator=g)).to(torch.float16).to(dev)
+    split = ops_fwd.linear_fwd(a, W)
+    plain = torch.empty_like(split)
+    _cabi.check(_cabi.lib().gmlp_linear_fwd(a.data_ptr(), W.data_ptr(), None, plain.data_ptr(), 48, 8192, 1024, 0,
+                                            None, 0, _cabi.stream_ptr(dev)))
+    ref = a.float().cpu() @ W.float().cpu().T
+    _close("split", split, ref)
+    _close("plain", plain, ref)
+    assert (split.float() - plain.float()).abs().max().item() < 1e-2
+
+
 OTHER_ACTS = ["gelu", "relu", "leaky_relu", "sigmoid", "tanh", "no_act"]
 
 

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"libgmlp.so does not export {name}"
     assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
-    assert lib.gmlp_abi_version() == 2
+    assert lib.gmlp_abi_version() == 3
 
 
 def _buf(nbytes=4096):
@@ -44,15 +44,15 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     _, a = _buf()
     err = lambda: lib.gmlp_last_error().decode()
     # NULL pointer
-    assert lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None) == -1 and "NULL" in err()
+    assert lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None, 0, None) == -1 and "NULL" in err()
     # bad dtype; float32 is not available for the skinny-M kernels
-    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 8, 8, 7, None) == -1 and "dtype" in err()
+    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 8, 8, 7, None, 0, None) == -1 and "dtype" in err()
     assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 256, 2, 0, None) == -2
     # shape: K not a multiple of 8, M < 1
-    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None) == -2 and "multiple of 8" in err()
+    assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None, 0, None) == -2 and "multiple of 8" in err()
     assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0, 0.0, 0, 0, None) == -2
     # alignment
-    assert lib.gmlp_linear_fwd(a + 2, a, None, a, 8, 8, 8, 0, None) == -3 and "aligned" in err()
+    assert lib.gmlp_linear_fwd(a + 2, a, None, a, 8, 8, 8, 0, None, 0, None) == -3 and "aligned" in err()
     # dropout probability outside [0, 1)
     assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, 1.0, 0, 0, None) == -1
     assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, -0.1, 0, 0, None) == -1
@@ -68,22 +68,30 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     for fn, args in [
         (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0, 0.0, 0, 0, None)),
         (lib.gmlp_gating_bwd, (a, a, a, a, None, 8, 8, 0, 0, 0.0, 0, 0, None)),
-        (lib.gmlp_dx_bwd, (a, a, a, a, None, 8, 8, 8, 0, None)),
+        (lib.gmlp_dx_bwd, (a, a, a, a, None, 8, 8, 8, 0, None, 0, None)),
         (lib.gmlp_dw_bwd, (a, None, a, 8, 8, 8, 0, None)),
         (lib.gmlp_colsum, (a, a, None, 8, 8, 0, None)),
     ]:
         assert fn(*args) == -1
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, 100, 0, 64, 0) == 64 * 64 * 4
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DECODE_FWD, 16, 8192, 28672, 0) == 0
+    # split reduction: asked for by short batches with a long reduction only, never for float32
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, 8192, 14336, 4096, 0) == 0
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DX_BWD, 8192, 4096, 14336, 0) == 0
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, 64, 28672, 8192, 2) == 0
+    n = lib.gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, 64, 28672, 8192, 0)
+    assert n > 0 and n % (64 * 8192 * 4) == 0 and 2 <= n // (64 * 8192 * 4) <= 16
+    n = lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DX_BWD, 300, 4096, 14336, 1)
+    assert n > 0 and n % (300 * 4096 * 4) == 0
 
 
 def test_error_codes_map_to_python_exceptions():
     lib = _cabi.lib()
     _, a = _buf()
     with pytest.raises(NotImplementedError, match="multiple of 8"):
-        _cabi.check(lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None))
+        _cabi.check(lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None, 0, None))
     with pytest.raises(ValueError, match="NULL"):
-        _cabi.check(lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None))
+        _cabi.check(lib.gmlp_linear_fwd(None, a, None, a, 8, 8, 8, 0, None, 0, None))
     with pytest.raises(TypeError, match="float16, bfloat16 or float32"):
         _cabi.dtype_code(torch.float64)
     assert [_cabi.dtype_code(t) for t in (torch.float16, torch.bfloat16, torch.float32)] == [0, 1, 2]

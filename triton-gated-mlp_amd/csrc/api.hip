@@ -107,6 +107,37 @@ int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large, 
   return gmlp::TILE_MEDIUM_FULL;
 }
 
+// Compute units of the current device.
+int num_cu() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+// Number of workgroups that should share one output tile of a rows x cols GEMM with `red_tiles`
+// 64-wide reduction tiles, or 1.  A GEMM with a few output tiles and a long reduction (down
+// projection and input gradient of a short batch) leaves most of the chip idle and is bound by
+// streaming the weights; splitting the reduction fills two 128-tile workgroups per CU.  Each split
+// keeps at least 8 reduction tiles.
+int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_tiles) {
+  if (pick_tile(dtype, rows, cols, red, 256) != gmlp::TILE_MEDIUM_FULL) return 1;
+  const int64_t tiles = ((rows + 127) / 128) * ((cols + 127) / 128);
+  int64_t s = 2 * num_cu() / tiles;
+  if (s > red_tiles / 8) s = red_tiles / 8;
+  if (s > 16) s = 16;
+  return s >= 2 ? (int)s : 1;
+}
+
+size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols) {
+  return splits > 1 ? (size_t)splits * rows * cols * sizeof(float) : 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -115,9 +146,13 @@ int gmlp_abi_version(void) { return GMLP_ABI_VERSION; }
 const char* gmlp_last_error(void) { return g_err; }
 
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {
-  (void)K;
-  (void)dtype;
-  if (op == GMLP_OP_COLSUM && M >= 1 && N >= 1) return gmlp::colsum_workspace_bytes(M, N);
+  if (M < 1 || N < 1) return 0;
+  if (op == GMLP_OP_COLSUM) return gmlp::colsum_workspace_bytes(M, N);
+  if (K < 1) return 0;
+  // gmlp_linear_fwd(M, R = K, C = N): out [M,N], reduction K
+  if (op == GMLP_OP_LINEAR_FWD) return split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64), M, N);
+  // gmlp_dx_bwd(M, K, N): out [M,K], reduction over two segments of N
+  if (op == GMLP_OP_DX_BWD) return split_workspace_bytes(pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64)), M, K);
   return 0;
 }
 
@@ -154,7 +189,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
 }
 
 int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, int64_t M, int64_t R,
-                    int64_t C, int dtype, void* stream) {
+                    int64_t C, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(w); GMLP_REQUIRE_PTR(out);
   GMLP_REQUIRE_DTYPE(dtype);
@@ -162,16 +197,26 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   if (int rc = check_mult8(__func__, "R", R)) return rc;
   if (int rc = check_mult8(__func__, "C", C)) return rc;
   GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(w); GMLP_REQUIRE_ALIGNED(bias);
-  GMLP_REQUIRE_ALIGNED(out);
+  GMLP_REQUIRE_ALIGNED(out); GMLP_REQUIRE_ALIGNED(workspace);
 
   GemmArgs ga = {};
   ga.A[0] = a; ga.A[1] = a; ga.B[0] = w; ga.B[1] = w;
   ga.M = (int)M; ga.N = (int)C; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(dtype, M, C, R, 256);
+  const int splits = pick_splits(dtype, M, C, R, (R + 63) / 64);
+  const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, C);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = by_dtype(dtype, [&](auto tag) {
+  hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
+    if constexpr (!std::is_same<T, float>::value) {
+      if (split) {
+        ga.splits = splits;
+        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * C, (int)C};
+        if (hipError_t err = launch_linear_split<T>(ga, pa, s)) return err;
+        return launch_splitk_reduce<T>((const float*)workspace, splits, (size_t)M * C, (const T*)bias, (T*)out, M, C, s);
+      }
+    }
     typename EpiStore<T>::Args ea = {(T*)out, (const T*)bias, (int)C};
     return launch_linear<T>(tc, ga, ea, s);
   });
@@ -232,7 +277,8 @@ int gmlp_gating_bwd(const void* dh, const void* g, const void* u, void* dg, void
 }
 
 int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* w_up, void* dx,
-                int64_t M, int64_t K, int64_t N, int dtype, void* stream) {
+                int64_t M, int64_t K, int64_t N, int dtype, void* workspace, size_t workspace_bytes,
+                void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(dg); GMLP_REQUIRE_PTR(du); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up);
   GMLP_REQUIRE_PTR(dx);
@@ -241,7 +287,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   if (int rc = check_mult8(__func__, "K", K)) return rc;
   if (int rc = check_mult8(__func__, "N", N)) return rc;
   GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du); GMLP_REQUIRE_ALIGNED(w_gate);
-  GMLP_REQUIRE_ALIGNED(w_up); GMLP_REQUIRE_ALIGNED(dx);
+  GMLP_REQUIRE_ALIGNED(w_up); GMLP_REQUIRE_ALIGNED(dx); GMLP_REQUIRE_ALIGNED(workspace);
 
   // dX[M,K] = dG[M,N]·W_gate[N,K] + dU[M,N]·W_up[N,K]: two reduction segments of length N.
   GemmArgs ga = {};
@@ -249,9 +295,19 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
   ga.nseg = 2; ga.group_m = 8;
   int tc = pick_tile(dtype, M, K, N, 256);
+  const int splits = pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64));
+  const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, K);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = by_dtype(dtype, [&](auto tag) {
+  hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
+    if constexpr (!std::is_same<T, float>::value) {
+      if (split) {
+        ga.splits = splits;
+        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * K, (int)K};
+        if (hipError_t err = launch_dx_split<T>(ga, pa, s)) return err;
+        return launch_splitk_reduce<T>((const float*)workspace, splits, (size_t)M * K, (const T*)nullptr, (T*)dx, M, K, s);
+      }
+    }
     typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};
     return launch_dx<T>(tc, ga, ea, s);
   });

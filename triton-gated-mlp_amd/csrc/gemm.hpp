@@ -26,17 +26,22 @@ struct GemmArgs {
   int lda, ldb;      // leading dimensions (elements)
   int nseg;          // number of reduction segments (1 or 2)
   int group_m;       // tile-rows per scheduling group
+  int splits;        // pipelined kernel with a split-reduction epilogue only: number of workgroups
+                     // that share one output tile, each reducing a contiguous range of 64-wide
+                     // reduction tiles into a partial result of its own (0 or 1: no split)
 };
 
 // Workgroup id -> output tile.  The hardware deals consecutive workgroup ids round-robin to the
-// 8 XCDs (each with its own L2); undo that so each XCD walks a contiguous run of tiles, then walk
-// tiles in groups of `group_m` tile-rows (column-major inside a group) for operand reuse in L2.
-__device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tiles_n, int group_m,
-                                         int& tm, int& tn) {
+// 8 XCDs (each with its own L2); xcd_contiguous undoes that so each XCD walks a contiguous run of
+// indices, and tile_of walks tiles in groups of `group_m` tile-rows (column-major inside a group)
+// for operand reuse in L2.
+__device__ __forceinline__ int xcd_contiguous(int pid, int nwg) {
   const int NXCD = 8;
   int xcd = pid % NXCD, loc = pid / NXCD;
   int per = nwg / NXCD, rem = nwg % NXCD;
-  int t = xcd * per + (xcd < rem ? xcd : rem) + loc;
+  return xcd * per + (xcd < rem ? xcd : rem) + loc;
+}
+__device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
   int in_group = group_m * tiles_n;
   int gid = t / in_group;
   int first_m = gid * group_m;
@@ -44,6 +49,10 @@ __device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tile
   int r = t - gid * in_group;
   tm = first_m + r % gsz;
   tn = r / gsz;
+}
+__device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tiles_n, int group_m,
+                                         int& tm, int& tn) {
+  tile_of(xcd_contiguous(pid, nwg), tiles_m, tiles_n, group_m, tm, tn);
 }
 
 template <int BK>
@@ -288,6 +297,7 @@ struct EpiStore {
   // Nothing worth fetching ahead of time (see EpiDh), no activation to specialise on.
   static constexpr int PREFETCH_DEPTH = 0;
   static constexpr bool HAS_ACT = false;
+  static constexpr bool SPLIT = false;
   template <int W>
   struct Prefetch {};
   template <int W>
@@ -296,6 +306,31 @@ struct EpiStore {
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float* w,
                                                const Prefetch<W>&) {
     apply<W>(a, m, n, v, w);
+  }
+};
+
+// Split reduction: workgroup `split` of an output tile stores its fp32 partial sums to
+// ws[split][m][n]; splitk_reduce (aux.hip) adds the partials up and applies EpiStore.
+template <typename T>
+struct EpiPartial {
+  struct Args {
+    float* ws;
+    size_t split_stride;  // elements between the partial results of consecutive splits
+    int ldc;
+  };
+  static constexpr int PREFETCH_DEPTH = 0;
+  static constexpr bool HAS_ACT = false;
+  static constexpr bool SPLIT = true;
+  template <int W>
+  struct Prefetch {};
+  template <int W>
+  static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
+  template <int W, int ACT>
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float*,
+                                               const Prefetch<W>&) {
+    float* p = a.ws + (size_t)m * a.ldc + n;
+#pragma unroll
+    for (int q = 0; q < W / 4; ++q) *(f32x4*)(p + 4 * q) = *(const f32x4*)(v + 4 * q);
   }
 };
 
@@ -317,6 +352,7 @@ struct EpiGateUp {
   // is unrolled many times instantiates both and branches once, so that the usual SiLU path stays
   // as compact as if it were the only one (HAS_ACT tells it that the choice exists).
   static constexpr bool HAS_ACT = true;
+  static constexpr bool SPLIT = false;
   template <int W, int ACT = ACT_RUNTIME>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* g, float* u) {
     if (a.b_gate) add_w<T, W>(a.b_gate + n, g);
@@ -421,6 +457,7 @@ struct EpiDh {
     p.u = *(const pack*)(a.u + e);
   }
   static constexpr bool HAS_ACT = true;
+  static constexpr bool SPLIT = false;
   template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*,
                                                const Prefetch<W>& p) {

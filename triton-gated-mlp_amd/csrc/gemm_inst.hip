@@ -38,6 +38,10 @@ hipError_t launch_linear<DT>(int tile_class, const GemmArgs& ga, const EpiStore<
                              hipStream_t s) {
   GMLP_DISPATCH(false, false, 1, EpiStore, 256, 128)
 }
+template <>
+hipError_t launch_linear_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
+  return launch_gemm_pipelined<DT, 128, 128, GMLP_MI, 2, 2, false, false, 1, EpiPartial<DT>>(ga, ea, s);
+}
 #elif GMLP_KIND == 2
 template <>
 hipError_t launch_dh<DT>(int tile_class, const GemmArgs& ga, const EpiDh<DT>::Args& ea,
@@ -49,6 +53,10 @@ template <>
 hipError_t launch_dx<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>::Args& ea,
                          hipStream_t s) {
   GMLP_DISPATCH(false, true, 1, EpiStore, 256, 128)
+}
+template <>
+hipError_t launch_dx_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
+  return launch_gemm_pipelined<DT, 128, 128, GMLP_MI, 2, 2, false, true, 1, EpiPartial<DT>>(ga, ea, s);
 }
 #elif GMLP_KIND == 4
 template <>

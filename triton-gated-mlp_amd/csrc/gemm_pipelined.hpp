@@ -82,8 +82,8 @@ struct PipeConfig {
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
           typename Epi>
-__device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const typename Epi::Args& ea,
-                                             int pid, int nwg) {
+__device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const typename Epi::Args& ea_in,
+                                                    int pid, int nwg) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
   typedef typename Cfg::ATile ATile;
   typedef typename Cfg::BTile BTile;
@@ -111,9 +111,15 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const int wm = wave / WGN, wn = wave % WGN;
 
   const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
+  // Workgroup -> (split, tile): all tiles of split 0, then all tiles of split 1, ...
+  const int ntiles = tiles_m * tiles_n;
+  const int u = xcd_contiguous(pid, nwg);
+  const int split = Epi::SPLIT ? u / ntiles : 0;
   int tm_i, tn_i;
-  map_tile(pid, nwg, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  tile_of(u - split * ntiles, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
   const int m0 = tm_i * BM, n0 = tn_i * BN;
+  typename Epi::Args ea = ea_in;
+  if constexpr (Epi::SPLIT) ea.ws += (size_t)split * ea.split_stride;
 
   acc_t acc[G][TM];
 #pragma unroll
@@ -123,8 +129,15 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 #pragma unroll
       for (int r = 0; r < (int)(sizeof(acc_t) / 4); ++r) acc[g][i][r] = 0.f;
 
+  // This workgroup reduces the 64-wide reduction tiles [kt_first, kt_total) of the concatenated
+  // segments: everything, or its share of a split reduction.
   const int kt_seg = (ga.K + BK - 1) / BK;
-  const int kt_total = kt_seg * ga.nseg;
+  int kt_first = 0, kt_total = kt_seg * ga.nseg;
+  if constexpr (Epi::SPLIT) {
+    const int per = (kt_total + ga.splits - 1) / ga.splits;
+    kt_first = split * per;
+    kt_total = kt_first + per < kt_total ? kt_first + per : kt_total;
+  }
 
   // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
   // Buffer addressing uses 32-bit byte offsets from each operand's base; the host checks sizes.
@@ -269,20 +282,20 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   constexpr int L_HEAD = HEAD_LOADS < L ? HEAD_LOADS : L;
 #pragma unroll
   for (int x = 0; x < L; ++x) {
-    if (starts_group(x)) dma_base(0, x);
-    issue_one(0, x);
+    if (starts_group(x)) dma_base(kt_first, x);
+    issue_one(kt_first, x);
   }
 #pragma unroll
   for (int x = 0; x < L_HEAD; ++x) {
-    if (starts_group(x)) dma_base(1, x);
-    issue_one(1, x);
+    if (starts_group(x)) dma_base(kt_first + 1, x);
+    issue_one(kt_first + 1, x);
   }
   wait_vmem<L_HEAD>();
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < TM; ++i) fetch_a(0, i, 0, 0);
+  for (int i = 0; i < TM; ++i) fetch_a(0, i, kt_first, 0);
 #pragma unroll
-  for (int g = 0; g < LA; ++g) fetch_b(g, g, 0, 0);
+  for (int g = 0; g < LA; ++g) fetch_b(g, g, kt_first, 0);
   __builtin_amdgcn_sched_barrier(0);
 
   // Epilogue work items of a wavefront: MI-row slab i of its tile, then (row, 8-column group)
@@ -303,7 +316,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   };
   typename Epi::template Prefetch<8> pf[PD > 0 ? PD : 1];
 
-  int kt = 0;
+  int kt = kt_first;
   for (; kt + 1 < kt_total; ++kt) tile_body(kt, std::true_type{});
 #pragma unroll
   for (int q = 0; q < PD; ++q) {
@@ -401,7 +414,8 @@ hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& e
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
-  dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN)), block(Cfg::NW * 64);
+  const int splits = Epi::SPLIT ? ga.splits : 1;
+  dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN) * splits), block(Cfg::NW * 64);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
   return hipGetLastError();
 }

@@ -46,6 +46,12 @@ hipError_t launch_gemm(const GemmArgs& ga, const typename Epi::Args& ea, hipStre
   return hipGetLastError();
 }
 
+// Split-reduction variants (128x128 tiles): partial sums to a fp32 workspace, see splitk_reduce.
+template <typename T>
+hipError_t launch_linear_split(const GemmArgs& ga, const typename EpiPartial<T>::Args& ea, hipStream_t s);
+template <typename T>
+hipError_t launch_dx_split(const GemmArgs& ga, const typename EpiPartial<T>::Args& ea, hipStream_t s);
+
 // decode.hip
 template <typename T>
 hipError_t launch_decode(const T* x, const T* wg, const T* wu, const T* wd, const T* bg,
@@ -63,6 +69,10 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
 template <typename T>
 hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
                              int act, const DropoutParams& d, hipStream_t s);
+// out[m,n] = sum_s ws[s*stride + m*N + n] (+ bias[n]): second stage of a split reduction
+template <typename T>
+hipError_t launch_splitk_reduce(const float* ws, int splits, size_t stride, const T* bias, T* out,
+                                int64_t M, int64_t N, hipStream_t s);
 template <typename T>
 hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s);
 size_t colsum_workspace_bytes(int64_t M, int64_t C);

@@ -15,8 +15,8 @@ import torch
 from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
-GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM = 0, 1
-ABI_VERSION = 2
+GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD = 0, 1, 2, 3
+ABI_VERSION = 3
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
 # tables (src/triton_gated_mlp/gated_mlp.py:17-37).
@@ -44,10 +44,10 @@ _SIGNATURES = {
     "gmlp_last_error": (ctypes.c_char_p, []),
     "gmlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
     "gmlp_gateup_fwd": (_int, [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
-    "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
     "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
     "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
-    "gmlp_dx_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _i64, _int, _c_ptr]),
+    "gmlp_dx_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
     "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr]),
     "gmlp_dw_bwd_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _c_ptr, _int, _c_ptr]),
     "gmlp_colsum": (_int, [_c_ptr] * 3 + [_i64, _i64, _int, _c_ptr]),
@@ -135,6 +135,12 @@ def require_gpu(*tensors: Optional[Tensor]) -> torch.device:
             raise TypeError(f"tensors of different dtypes: {dt} and {t.dtype}")
     assert dev is not None
     return dev
+
+
+def workspace(op: int, M: int, K: int, N: int, code: int, device: torch.device) -> Optional[Tensor]:
+    """Scratch buffer of the size the library asks for (None if it needs none)."""
+    nbytes = lib().gmlp_workspace_bytes(op, M, K, N, code)
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device) if nbytes else None
 
 
 def ptr(t: Optional[Tensor]) -> Optional[int]:

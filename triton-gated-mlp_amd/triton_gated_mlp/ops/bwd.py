@@ -91,10 +91,11 @@ def dx_bwd(dg: Tensor, du: Tensor, W_gate: Tensor, W_up: Tensor) -> Tensor:
     dx = torch.empty((M, K), dtype=dg.dtype, device=dev)
     if M > 0:
         with torch.cuda.device(dev):
+            ws = _cabi.workspace(_cabi.GMLP_OP_DX_BWD, M, K, N, code, dev)
             _cabi.check(
                 _cabi.lib().gmlp_dx_bwd(
                     _cabi.ptr(dg), _cabi.ptr(du), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(dx), M, K, N,
-                    code, _cabi.stream_ptr(dev),
+                    code, _cabi.ptr(ws), 0 if ws is None else ws.numel(), _cabi.stream_ptr(dev),
                 )
             )
     return dx

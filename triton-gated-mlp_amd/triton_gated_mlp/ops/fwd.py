@@ -115,10 +115,11 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
     out = torch.empty((M, C), dtype=a.dtype, device=dev)
     if M > 0:
         with torch.cuda.device(dev):
+            ws = _cabi.workspace(_cabi.GMLP_OP_LINEAR_FWD, M, R, C, code, dev)
             _cabi.check(
                 _cabi.lib().gmlp_linear_fwd(
                     _cabi.ptr(a), _cabi.ptr(W), _cabi.ptr(bias), _cabi.ptr(out), M, R, C, code,
-                    _cabi.stream_ptr(dev),
+                    _cabi.ptr(ws), 0 if ws is None else ws.numel(), _cabi.stream_ptr(dev),
                 )
             )
     return out
