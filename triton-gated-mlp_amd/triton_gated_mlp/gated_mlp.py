@@ -231,7 +231,9 @@ class FusedGatedMLP(_GatedMLPBase):
         inference = not torch.is_grad_enabled() or not (
             x2.requires_grad or any(q.requires_grad for q in self.parameters())
         )
-        if inference and p == 0.0 and _fwd.decode_supported(M, K, self.intermediate_size, x2.dtype):
+        if inference and p == 0.0 and x2.is_cuda and _fwd.decode_preferred(
+            M, K, self.intermediate_size, x2.dtype, torch.cuda.get_device_properties(x2.device).multi_processor_count
+        ):
             y = _fwd.decode_fwd(
                 x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, self.act_fn
             )
