@@ -86,27 +86,6 @@ int hip_result(const char* fn, hipError_t e) {
   return fail(GMLP_EHIP, "%s: HIP error %d (%s)", fn, (int)e, hipGetErrorString(e));
 }
 
-// Tile class for an output of rows x cols with reduction length red (all in elements).
-// The pipelined kernels (LARGE: 256 x bn_large tiles, one workgroup per CU; MEDIUM_FULL: tiles of
-// half that in each direction, two per CU) take any rows and cols; they need 32-bit byte offsets
-// into the operands, padded to whole tiles, and a reduction that is a multiple of 64 unless both
-// operands are reduction-strided (`both_ks`).  Everything else runs on the predicated MEDIUM class.
-// Between the two pipelined classes the choice is padded work, with the small tiles counted at
-// the 75 % of the large tiles' throughput they reach, and enough large tiles to occupy the chip.
-int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large, bool both_ks = false) {
-  if (dtype == GMLP_F32) return gmlp::TILE_MEDIUM;  // the float32 kernel has one tile shape
-  auto up = [](int64_t v, int64_t q) { return (v + q - 1) / q * q; };
-  // the buffer base sits up to 4 KB below the operand (shared-M0 loads)
-  const int64_t limit = ((int64_t)1 << 31) - 4096;
-  bool offsets_fit = up(rows, 256) * up(red, 64) * 2 < limit && up(cols, 256) * up(red, 64) * 2 < limit;
-  if (!offsets_fit || (red % 64 != 0 && !both_ks)) return gmlp::TILE_MEDIUM;
-  const int64_t large_tiles = (up(rows, 256) / 256) * (up(cols, bn_large) / bn_large);
-  const double large_work = (double)up(rows, 256) * up(cols, bn_large);
-  const double medium_work = (double)up(rows, 128) * up(cols, bn_large / 2) / 0.75;
-  if (large_tiles >= 192 && large_work <= medium_work) return gmlp::TILE_LARGE;
-  return gmlp::TILE_MEDIUM_FULL;
-}
-
 // Compute units of the current device.
 int num_cu() {
   static int cached[64] = {};
@@ -118,6 +97,40 @@ int num_cu() {
     cached[dev] = n;
   }
   return cached[dev];
+}
+
+// LARGE or MEDIUM_FULL for a grid of `large_tiles` large or `medium_tiles` small tiles, by
+// estimated time in rounds of workgroups (see pick_tile).
+int group_tile_class(int64_t large_tiles, int64_t medium_tiles) {
+  auto rounds = [](int64_t tiles, int64_t slots) {
+    double part = (double)(tiles % slots) / (double)slots;
+    return (double)(tiles / slots) + (part > 0.0 ? 0.6 + 0.4 * part : 0.0);
+  };
+  const int64_t cus = num_cu();
+  const double large_time = rounds(large_tiles, cus);
+  const double medium_time = rounds(medium_tiles, 2 * cus) * (2.0 / 3.0);
+  return large_time <= medium_time ? gmlp::TILE_LARGE : gmlp::TILE_MEDIUM_FULL;
+}
+
+// Tile class for an output of rows x cols with reduction length red (all in elements).
+// The pipelined kernels (LARGE: 256 x bn_large tiles, one workgroup per CU; MEDIUM_FULL: tiles of
+// half that in each direction, two per CU) take any rows and cols; they need 32-bit byte offsets
+// into the operands, padded to whole tiles, and a reduction that is a multiple of 64 unless both
+// operands are reduction-strided (`both_ks`).  Everything else runs on the predicated MEDIUM class.
+// Between the two pipelined classes the choice is estimated time in rounds of workgroups: a round
+// of small tiles (two per CU) takes 2/3 of a round of large ones (a quarter of the work at 75 % of
+// the throughput, two at a time), and a last round filled to the fraction f costs 0.6 + 0.4 f of
+// a full one (the busy CUs clock higher, but not in proportion; fitted to measurements).
+int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large, bool both_ks = false) {
+  if (dtype == GMLP_F32) return gmlp::TILE_MEDIUM;  // the float32 kernel has one tile shape
+  auto up = [](int64_t v, int64_t q) { return (v + q - 1) / q * q; };
+  // the buffer base sits up to 4 KB below the operand (shared-M0 loads)
+  const int64_t limit = ((int64_t)1 << 31) - 4096;
+  bool offsets_fit = up(rows, 256) * up(red, 64) * 2 < limit && up(cols, 256) * up(red, 64) * 2 < limit;
+  if (!offsets_fit || (red % 64 != 0 && !both_ks)) return gmlp::TILE_MEDIUM;
+  const int64_t large_tiles = (up(rows, 256) / 256) * (up(cols, bn_large) / bn_large);
+  const int64_t medium_tiles = (up(rows, 128) / 128) * (up(cols, bn_large / 2) / (bn_large / 2));
+  return group_tile_class(large_tiles, medium_tiles);
 }
 
 // Number of workgroups that should share one output tile of a rows x cols GEMM with `red_tiles`
@@ -347,20 +360,28 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
   GMLP_REQUIRE_PTR(lhs); GMLP_REQUIRE_PTR(rhs); GMLP_REQUIRE_PTR(dw); GMLP_REQUIRE_PTR(R);
   GMLP_REQUIRE_PTR(C);
   GMLP_REQUIRE_DTYPE(dtype);
-  bool large = true;
+  // One grid when every problem runs on a pipelined tile class; the class is chosen for the
+  // problems together (their tiles share the rounds of workgroups).
+  bool pipelined = true;
   for (int i = 0; i < count; ++i) {
     GMLP_REQUIRE_PTR(lhs[i]); GMLP_REQUIRE_PTR(rhs[i]); GMLP_REQUIRE_PTR(dw[i]);
     if (int rc = check_dims(__func__, Mred, R[i], C[i])) return rc;
     if (int rc = check_mult8(__func__, "R", R[i])) return rc;
     if (int rc = check_mult8(__func__, "C", C[i])) return rc;
     GMLP_REQUIRE_ALIGNED(lhs[i]); GMLP_REQUIRE_ALIGNED(rhs[i]); GMLP_REQUIRE_ALIGNED(dw[i]);
-    large = large && pick_tile(dtype, R[i], C[i], Mred, 256, true) == TILE_LARGE;
+    pipelined = pipelined && pick_tile(dtype, R[i], C[i], Mred, 256, true) != TILE_MEDIUM;
   }
-  if (!large) {
+  if (!pipelined) {
     for (int i = 0; i < count; ++i)
       if (int rc = gmlp_dw_bwd(lhs[i], rhs[i], dw[i], Mred, R[i], C[i], dtype, stream)) return rc;
     return GMLP_OK;
   }
+  int64_t tiles256 = 0, tiles128 = 0;
+  for (int i = 0; i < count; ++i) {
+    tiles256 += ((R[i] + 255) / 256) * ((C[i] + 255) / 256);
+    tiles128 += ((R[i] + 127) / 128) * ((C[i] + 127) / 128);
+  }
+  const int group_class = group_tile_class(tiles256, tiles128);
   hipStream_t s = (hipStream_t)stream;
   auto fill = [&](GemmArgs& ga, int i) {
     ga = GemmArgs{};
@@ -379,7 +400,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
         fill(grp.ga[i], i);
         grp.ea[i] = typename EpiStore<T>::Args{(T*)dw[i], nullptr, (int)C[i]};
       }
-      return launch_dw_group<T>(grp, s);
+      return launch_dw_group<T>(group_class, grp, s);
     }
   });
   return hip_result(__func__, e);

@@ -20,6 +20,8 @@ typedef bf16 DT;
   launch_gemm_pipelined<DT, 128, BN_M, GMLP_MI, 2, 2, AKS, BKS, NB, EPI<DT>>
 #define GMLP_LARGE_GROUP \
   launch_gemm_group_pipelined<DT, 256, 256, GMLP_MI, 2, 2, true, true, 1, EpiStore<DT>>
+#define GMLP_MEDIUM_GROUP \
+  launch_gemm_group_pipelined<DT, 128, 128, GMLP_MI, 2, 2, true, true, 1, EpiStore<DT>>
 
 #define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
   if (tile_class == TILE_LARGE) return GMLP_LARGE(AKS, BKS, NB, EPI, BN_L)(ga, ea, s);           \
@@ -65,8 +67,8 @@ hipError_t launch_dw<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>:
   GMLP_DISPATCH(true, true, 1, EpiStore, 256, 128)
 }
 template <>
-hipError_t launch_dw_group<DT>(GemmGroup<EpiStore<DT>::Args>& grp, hipStream_t s) {
-  return GMLP_LARGE_GROUP(grp, s);
+hipError_t launch_dw_group<DT>(int tile_class, GemmGroup<EpiStore<DT>::Args>& grp, hipStream_t s) {
+  return tile_class == TILE_LARGE ? GMLP_LARGE_GROUP(grp, s) : GMLP_MEDIUM_GROUP(grp, s);
 }
 #endif
 

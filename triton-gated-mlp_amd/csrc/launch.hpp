@@ -29,9 +29,9 @@ template <typename T>
 hipError_t launch_dw(int tile_class, const GemmArgs& ga, const typename EpiStore<T>::Args& ea,
                      hipStream_t s);  // A KS, B KS
 
-// Several LARGE-class weight-gradient GEMMs (every problem: whole 256x256 tiles, Mred % 64 == 0).
+// Several weight-gradient GEMMs of one pipelined tile class (LARGE or MEDIUM_FULL) as one grid.
 template <typename T>
-hipError_t launch_dw_group(GemmGroup<typename EpiStore<T>::Args>& grp, hipStream_t s);
+hipError_t launch_dw_group(int tile_class, GemmGroup<typename EpiStore<T>::Args>& grp, hipStream_t s);
 
 // Generic launcher used by the instantiation units.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
