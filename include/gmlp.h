@@ -158,6 +158,14 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
                 void* stream);
 
 /*
+ * Up to 3 bias gradients of one backward pass in one pair of launches: out[i][C[i]] = Σ_m a[i][m,C[i]].
+ * workspace: the sum over i of gmlp_workspace_bytes(GMLP_OP_COLSUM, M, 0, C[i], dtype) bytes.
+ * Same reference counterpart as gmlp_colsum.
+ */
+int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void* workspace, int64_t M,
+                        const int64_t* C, int dtype, void* stream);
+
+/*
  * Skinny-M forward of the whole MLP (decode): y = (act(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
  * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch is [M,N] in dtype;
  * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).

@@ -408,16 +408,38 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
 
 int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C, int dtype,
                 void* stream) {
+  const void* as[1] = {a};
+  void* outs[1] = {out};
+  return gmlp_colsum_grouped(1, as, outs, workspace, M, &C, dtype, stream);
+}
+
+int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void* workspace, int64_t M,
+                        const int64_t* C, int dtype, void* stream) {
   using namespace gmlp;
-  GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(out); GMLP_REQUIRE_PTR(workspace);
+  if (count < 1 || count > COLSUM_GROUP_MAX)
+    return fail(GMLP_EINVAL, "%s: count = %d must be in 1..%d", __func__, count, COLSUM_GROUP_MAX);
+  GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(out); GMLP_REQUIRE_PTR(C); GMLP_REQUIRE_PTR(workspace);
   GMLP_REQUIRE_DTYPE(dtype);
-  if (int rc = check_dims(__func__, M, 8, C)) return rc;
-  if (int rc = check_mult8(__func__, "C", C)) return rc;
-  GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(out); GMLP_REQUIRE_ALIGNED(workspace);
+  GMLP_REQUIRE_ALIGNED(workspace);
+  for (int i = 0; i < count; ++i) {
+    GMLP_REQUIRE_PTR(a[i]); GMLP_REQUIRE_PTR(out[i]);
+    if (int rc = check_dims(__func__, M, 8, C[i])) return rc;
+    if (int rc = check_mult8(__func__, "C", C[i])) return rc;
+    GMLP_REQUIRE_ALIGNED(a[i]); GMLP_REQUIRE_ALIGNED(out[i]);
+  }
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
-    return launch_colsum<T>((const T*)a, (T*)out, (float*)workspace, M, C, s);
+    ColsumGroup<T> g = {};
+    char* ws = (char*)workspace;
+    for (int i = 0; i < count; ++i) {
+      g.a[i] = (const T*)a[i];
+      g.out[i] = (T*)out[i];
+      g.ws[i] = (float*)ws;
+      g.C[i] = C[i];
+      ws += colsum_workspace_bytes(M, C[i]);
+    }
+    return launch_colsum_group<T>(g, count, M, s);
   });
   return hip_result(__func__, e);
 }

@@ -77,50 +77,69 @@ template hipError_t launch_splitk_reduce<bf16>(const float*, int, size_t, const 
                                                int64_t, hipStream_t);
 
 // Column sums in two fixed-order stages: COLSUM_SPLITS row ranges -> fp32 partials -> total.
+// Up to COLSUM_GROUP_MAX arrays with the same number of rows share the two launches (the bias
+// gradients of one backward pass); blockIdx.z selects the array.
 constexpr int COLSUM_SPLITS = 64;
 
 template <typename T>
-__global__ void __launch_bounds__(256)
-    colsum_partial_kernel(const T* __restrict__ a, float* __restrict__ ws, int64_t M, int64_t C) {
-  int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+__global__ void __launch_bounds__(256) colsum_partial_kernel(ColsumGroup<T> g, int64_t M) {
+  const T* __restrict__ a = g.a[blockIdx.z];
+  float* __restrict__ ws = g.ws[blockIdx.z];
+  const int64_t C = g.C[blockIdx.z];
+  int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (c >= C) return;
   int64_t rows = (M + COLSUM_SPLITS - 1) / COLSUM_SPLITS;
   int64_t r0 = blockIdx.y * rows, r1 = r0 + rows < M ? r0 + rows : M;
-  f32x4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t r = r0; r < r1; ++r) {
-    float t[4];
-    load_w<T, 4>(a + r * C + c, t);
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  int64_t r = r0;
+  for (; r + 4 <= r1; r += 4) {  // four independent 16-byte loads in flight per lane
+    float t[4][8];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) s[q] += t[q];
+    for (int u = 0; u < 4; ++u) load_w<T, 8>(a + (r + u) * C + c, t[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int q = 0; q < 8; ++q) s[q] += t[u][q];
   }
-  *(f32x4*)(ws + (int64_t)blockIdx.y * C + c) = s;
+  for (; r < r1; ++r) {
+    float t[8];
+    load_w<T, 8>(a + r * C + c, t);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) s[q] += t[q];
+  }
+  float* p = ws + (int64_t)blockIdx.y * C + c;
+  *(f32x4*)p = f32x4{s[0], s[1], s[2], s[3]};
+  *(f32x4*)(p + 4) = f32x4{s[4], s[5], s[6], s[7]};
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256)
-    colsum_final_kernel(const float* __restrict__ ws, T* __restrict__ out, int64_t C) {
+__global__ void __launch_bounds__(256) colsum_final_kernel(ColsumGroup<T> g) {
+  const float* __restrict__ ws = g.ws[blockIdx.z];
+  const int64_t C = g.C[blockIdx.z];
   int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (c >= C) return;
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
   for (int i = 0; i < COLSUM_SPLITS; ++i) s += *(const f32x4*)(ws + (int64_t)i * C + c);
   float t[4] = {s[0], s[1], s[2], s[3]};
-  store_w<T, 4>(out + c, t);
+  store_w<T, 4>(g.out[blockIdx.z] + c, t);
 }
 
 size_t colsum_workspace_bytes(int64_t, int64_t C) { return (size_t)COLSUM_SPLITS * C * sizeof(float); }
 
 template <typename T>
-hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s) {
-  unsigned bx = (unsigned)((C / 4 + 255) / 256);
-  hipLaunchKernelGGL(colsum_partial_kernel<T>, dim3(bx, COLSUM_SPLITS), dim3(256), 0, s, a, ws, M, C);
+hipError_t launch_colsum_group(const ColsumGroup<T>& g, int count, int64_t M, hipStream_t s) {
+  int64_t cmax = 0;
+  for (int i = 0; i < count; ++i) cmax = g.C[i] > cmax ? g.C[i] : cmax;
+  unsigned bx8 = (unsigned)((cmax / 8 + 255) / 256), bx4 = (unsigned)((cmax / 4 + 255) / 256);
+  hipLaunchKernelGGL(colsum_partial_kernel<T>, dim3(bx8, COLSUM_SPLITS, count), dim3(256), 0, s, g, M);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(colsum_final_kernel<T>, dim3(bx), dim3(256), 0, s, ws, out, C);
+  hipLaunchKernelGGL(colsum_final_kernel<T>, dim3(bx4, 1, count), dim3(256), 0, s, g);
   return hipGetLastError();
 }
-template hipError_t launch_colsum<f16>(const f16*, f16*, float*, int64_t, int64_t, hipStream_t);
-template hipError_t launch_colsum<bf16>(const bf16*, bf16*, float*, int64_t, int64_t, hipStream_t);
-template hipError_t launch_colsum<float>(const float*, float*, float*, int64_t, int64_t, hipStream_t);
+template hipError_t launch_colsum_group<f16>(const ColsumGroup<f16>&, int, int64_t, hipStream_t);
+template hipError_t launch_colsum_group<bf16>(const ColsumGroup<bf16>&, int, int64_t, hipStream_t);
+template hipError_t launch_colsum_group<float>(const ColsumGroup<float>&, int, int64_t, hipStream_t);
 
 __global__ void __launch_bounds__(256)
     dropout_mask_kernel(uint8_t* __restrict__ mask, size_t n4, DropoutParams d) {

@@ -73,8 +73,16 @@ hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, 
 template <typename T>
 hipError_t launch_splitk_reduce(const float* ws, int splits, size_t stride, const T* bias, T* out,
                                 int64_t M, int64_t N, hipStream_t s);
+constexpr int COLSUM_GROUP_MAX = 3;
 template <typename T>
-hipError_t launch_colsum(const T* a, T* out, float* ws, int64_t M, int64_t C, hipStream_t s);
+struct ColsumGroup {
+  const T* a[COLSUM_GROUP_MAX];   // [M, C[i]]
+  T* out[COLSUM_GROUP_MAX];       // [C[i]]
+  float* ws[COLSUM_GROUP_MAX];    // colsum_workspace_bytes(M, C[i]) bytes each
+  int64_t C[COLSUM_GROUP_MAX];
+};
+template <typename T>
+hipError_t launch_colsum_group(const ColsumGroup<T>& g, int count, int64_t M, hipStream_t s);
 size_t colsum_workspace_bytes(int64_t M, int64_t C);
 hipError_t launch_dropout_mask(uint8_t* mask, int64_t M, int64_t N, const DropoutParams& d,
                                hipStream_t s);

@@ -171,6 +171,7 @@ class FusedGatedMLPFullFunction(Function):
         dy = dy.contiguous()
         dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
         dw_jobs = []  # (slot, lhs, rhs): the weight gradients go out as one grouped launch
+        db_jobs = []  # (slot, array): so do the bias gradients
         if any(need[:5]):
             dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset, ctx.act_fn)
             if need[0]:
@@ -178,18 +179,21 @@ class FusedGatedMLPFullFunction(Function):
             if need[1]:
                 dw_jobs.append(("gate", dg, x))
             if ctx.has_bias[0] and need[2]:
-                db_gate = _bwd.colsum(dg)
+                db_jobs.append(("gate", dg))
             if need[3]:
                 dw_jobs.append(("up", du, x))
             if ctx.has_bias[1] and need[4]:
-                db_up = _bwd.colsum(du)
+                db_jobs.append(("up", du))
         if need[5]:
             dw_jobs.append(("down", dy, hidden))
+        if ctx.has_bias[2] and need[6]:
+            db_jobs.append(("down", dy))
         if dw_jobs:
             grads = dict(zip([j[0] for j in dw_jobs], _bwd.dw_bwd_grouped([(j[1], j[2]) for j in dw_jobs])))
             dW_gate, dW_up, dW_down = grads.get("gate"), grads.get("up"), grads.get("down")
-        if ctx.has_bias[2] and need[6]:
-            db_down = _bwd.colsum(dy)
+        if db_jobs:
+            grads = dict(zip([j[0] for j in db_jobs], _bwd.colsum_grouped([j[1] for j in db_jobs])))
+            db_gate, db_up, db_down = grads.get("gate"), grads.get("up"), grads.get("down")
         return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None, None, None
 
 

@@ -177,6 +177,40 @@ def colsum(a: Tensor) -> Tensor:
     return out
 
 
+def colsum_grouped(arrays):
+    """[Σ_m a[m,:] for a in arrays] (at most 3 arrays with the same number of rows) in one pair of
+    launches: the bias gradients of one backward pass."""
+    import ctypes
+
+    arrays = [_c(a) for a in arrays]
+    if not 1 <= len(arrays) <= 3:
+        raise ValueError("colsum_grouped takes 1 to 3 arrays")
+    M = arrays[0].shape[0]
+    for a in arrays:
+        if a.ndim != 2 or a.shape[0] != M:
+            raise ValueError("every array must be 2-D with the same number of rows")
+    dev = _cabi.require_gpu(*arrays)
+    code = _cabi.dtype_code(arrays[0].dtype)
+    if M == 0:
+        return [torch.zeros((a.shape[1],), dtype=a.dtype, device=dev) for a in arrays]
+    outs = [torch.empty((a.shape[1],), dtype=a.dtype, device=dev) for a in arrays]
+    n = len(arrays)
+    nbytes = sum(_cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, M, 0, a.shape[1], code) for a in arrays)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    PtrArr, I64Arr = ctypes.c_void_p * n, ctypes.c_int64 * n
+    srcs = PtrArr(*[a.data_ptr() for a in arrays])
+    dsts = PtrArr(*[o.data_ptr() for o in outs])
+    C = I64Arr(*[a.shape[1] for a in arrays])
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_colsum_grouped(
+                n, ctypes.cast(srcs, ctypes.c_void_p), ctypes.cast(dsts, ctypes.c_void_p), _cabi.ptr(ws), M,
+                ctypes.cast(C, ctypes.c_void_p), code, _cabi.stream_ptr(dev),
+            )
+        )
+    return outs
+
+
 def mlp_hidden_states_bwd(
     x: Tensor,
     W_up: Tensor,
@@ -205,5 +239,6 @@ def mlp_hidden_states_bwd(
     dW_up = dw_bwd(du, x)
     dW_gp = dw_bwd(dg, x)
     if return_bias_grads:
-        return dx, dW_up, colsum(du), dW_gp, colsum(dg)
+        db_up, db_gp = colsum_grouped([du, dg])
+        return dx, dW_up, db_up, dW_gp, db_gp
     return dx, dW_up, dW_gp
