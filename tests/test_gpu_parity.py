@@ -155,6 +155,7 @@ def test_ragged_token_counts_on_the_pipelined_kernels(M, K, N, dtype, bias, p):
         (64, 1024, 4096, torch.float16, False),
         (300, 1024, 4096, torch.bfloat16, True),
         (130, 4096, 14336, torch.float16, False),  # Llama-3-8B widths, short batch
+        (40, 1024, 4160, torch.float16, False),  # 130 reduction tiles for dX do not divide by 16 splits
     ],
 )
 def test_short_batches_split_the_long_reductions(M, K, N, dtype, bias):

@@ -144,7 +144,11 @@ int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_
   int64_t s = 2 * num_cu() / tiles;
   if (s > red_tiles / 8) s = red_tiles / 8;
   if (s > 16) s = 16;
-  return s >= 2 ? (int)s : 1;
+  if (s < 2) return 1;
+  // the kernel gives every split ceil(red_tiles / s) reduction tiles: drop the splits that this
+  // leaves empty
+  const int64_t per = (red_tiles + s - 1) / s;
+  return (int)((red_tiles + per - 1) / per);
 }
 
 size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols) {
