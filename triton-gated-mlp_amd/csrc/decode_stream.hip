@@ -221,7 +221,8 @@ template <typename T, bool GATED>
 static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
   constexpr int LDS = DS_WAVES * DS_RD * 2 * DS_REGION + 2 * (DS_WAVES - 1) * 2 * 256 * 4;
   auto kern = decode_stream_kernel<T, GATED>;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS)) return e;
+  static LdsAttrOnce lds_attr;
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
   int nblocks = a.R / (GATED ? 16 : 32);
   int grid = nblocks < num_cu ? nblocks : num_cu;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);

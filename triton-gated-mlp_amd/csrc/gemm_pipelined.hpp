@@ -413,7 +413,8 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
 hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
+  static LdsAttrOnce lds_attr;
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES, lds_attr)) return e;
   const int splits = Epi::SPLIT ? ga.splits : 1;
   dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN) * splits), block(Cfg::NW * 64);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
@@ -425,7 +426,8 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
 hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
   auto kern = gemm_group_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES)) return e;
+  static LdsAttrOnce lds_attr;
+  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES, lds_attr)) return e;
   int total = 0;
   for (int g = 0; g < grp.count; ++g) {
     grp.first[g] = total;

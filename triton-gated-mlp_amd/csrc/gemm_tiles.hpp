@@ -8,6 +8,7 @@
 // ds_read_b64_tr_b16, which hands each lane 4 consecutive reduction elements of one output row
 // out of a [k][row] tile.
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "gemm.hpp"
@@ -84,10 +85,21 @@ struct LdsTile {
   }
 };
 
-// Raises the dynamic-LDS limit of `kernel` on the current device (needed above 64 KiB).  Called on
-// every launch: the attribute is per device, and the call only touches host-side state.
-inline hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
-  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+// Raises the dynamic-LDS limit of `kernel` (needed above 64 KiB) the first time the kernel is
+// launched on a device; the attribute is per device and per kernel, so every launch site keeps a
+// flag array of its own.  After the first launch no runtime call but hipGetDevice is made, which
+// also keeps the launch path free of attribute calls while a stream is being captured.
+struct LdsAttrOnce {
+  std::atomic<unsigned char> done[64];
+};
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, LdsAttrOnce& once) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (tracked && once.done[dev].load(std::memory_order_acquire)) return hipSuccess;
+  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes)) return e;
+  if (tracked) once.done[dev].store(1, std::memory_order_release);
+  return hipSuccess;
 }
 
 // Up to GEMM_GROUP_MAX independent GEMMs of one kind in a single launch: workgroups
