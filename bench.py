@@ -141,6 +141,45 @@ def _other_configs(dev):
         flop = (18.0 if bwd else 6.0) * m * n * k
         out[name] = {"ms": round(med, 4), "tflops": round(flop / med / 1e9, 1),
                      "frac_mfma_peak": round(flop / med / 1e9 / PEAK_MFMA_F16_TFLOPS, 4)}
+        del mlp, x, dy, params
+    out.update(_edge_shapes(dev))
+    return out
+
+
+def _edge_shapes(dev):
+    """Shapes off the tile grid, next to torch's own operators (rocBLAS/hipBLASLt) on the same GPU:
+    a ragged token count at the headline widths (fwd+bwd) and a short batch at the decode widths
+    (forward; the down projection splits its reduction)."""
+    from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP
+
+    out = {}
+    for name, (m, k, n, bwd) in {
+        "ragged_fp16_fwdbwd_M8191_K4096_N14336": (8191, 4096, 14336, True),
+        "short_batch_fp16_fwd_M32_K8192_N28672": (32, 8192, 28672, False),
+    }.items():
+        fused = FusedGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
+        eager = EagerGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
+        x = torch.randn(m, k, device=dev, dtype=DTYPE, requires_grad=bwd)
+        dy = torch.randn(m, k, device=dev, dtype=DTYPE)
+        res = {}
+        for label, mod in (("ms", fused), ("torch_eager_ms", eager)):
+            params = list(mod.parameters())
+
+            def step():
+                if bwd:
+                    x.grad = None
+                    for q in params:
+                        q.grad = None
+                    mod(x).backward(dy)
+                else:
+                    with torch.no_grad():
+                        mod(x)
+
+            res[label] = round(_event_time_ms(step, 10, warmup=3)[1], 4)
+        flop = (18.0 if bwd else 6.0) * m * n * k
+        res["tflops"] = round(flop / res["ms"] / 1e9, 1)
+        out[name] = res
+        del fused, eager, x, dy
     return out
 
 
