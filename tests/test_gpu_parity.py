@@ -402,6 +402,11 @@ def test_reference_fp32_operator_forward():
     ref = eager_fwd(x, m.up_proj.weight, None, m.gate_proj.weight, None)
     out = mlp_hidden_states_fwd(x, m.up_proj.weight, None, m.gate_proj.weight, None, m.act_fn, m.dropout.p)
     assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+    # the reference builds this test's module with hidden_act="no_act" (tests/test_gated_mlp_fwd.py:41-82)
+    up = torch.nn.functional.linear(x, m.up_proj.weight)
+    gate = torch.nn.functional.linear(x, m.gate_proj.weight)
+    out = mlp_hidden_states_fwd(x, m.up_proj.weight, None, m.gate_proj.weight, None, "no_act", 0.0)
+    assert torch.allclose(out, gate * up, rtol=1e-4, atol=1e-5)
 
 
 def test_reference_fp32_module_backward_3d_input():
