@@ -3,7 +3,8 @@
 //
 // One persistent workgroup of three wavefronts per CU.  The workgroup owns blocks of 2 x 16 weight
 // rows (rb = blockIdx.x, blockIdx.x + gridDim.x, ...) that share one set of token operands: rows
-// r..r+15 of W_gate and of W_up (GATED), or 32 consecutive rows of W_down; its wavefronts split the reduction range in
+// r..r+15 of W_gate and of W_up (GATED), or 32 consecutive rows of W_down (16 when the hidden size
+// gives fewer than one 32-row block per CU); its wavefronts split the reduction range in
 // near-equal runs of 256-element chunks and combine their partial sums through LDS at the
 // end of each block (fixed order, so the result is deterministic).  Each wavefront runs a private
 // ring of 3 LDS slots; a slot holds one stage = 256 reduction elements of the 16 weight rows of
@@ -46,7 +47,8 @@ struct Mfma16x<bf16> {
 
 constexpr int DS_CH = 256;            // reduction elements per stage
 constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
-constexpr int DS_RD = 3;              // ring slots per wavefront (and stages in flight)
+// ring slots per wavefront (and stages in flight): 3 slots of two 16-row regions, or 4 of one
+constexpr int ds_ring_depth(int nmat) { return nmat == 2 ? 3 : 4; }
 constexpr int DS_WAVES = 3;           // wavefronts per workgroup
 
 struct StreamArgs {
@@ -80,11 +82,13 @@ __device__ __forceinline__ void wait_vmem_keep(i32x4 (&x)[8]) {
                : "memory");
 }
 
-template <typename T, bool GATED>
+// NMAT: 16-row regions per stage (GATED: W_gate and W_up; otherwise 1 or 2 runs of W_down rows).
+template <typename T, bool GATED, int NMAT>
 __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs a) {
   typedef typename Traits<T>::vec8 vec8;
-  constexpr int NMAT = 2;                       // 16-row regions per stage
-  constexpr int BLOCK_ROWS = GATED ? 16 : 32;   // weight rows (per matrix) a block advances by
+  static_assert(NMAT == 2 || (NMAT == 1 && !GATED), "gated blocks stream two matrices");
+  constexpr int DS_RD = ds_ring_depth(NMAT);
+  constexpr int BLOCK_ROWS = GATED ? 16 : 16 * NMAT;  // weight rows (per matrix) a block advances by
   constexpr int SLOT = NMAT * DS_REGION;
   constexpr int LPS = 8 + 8 * NMAT;  // load instructions per stage (token operands + weights)
   static_assert((DS_RD - 1) * LPS < 64, "the younger stages must fit the 6-bit vmcnt");
@@ -200,11 +204,11 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
               float res[4];
               act_fwd_w<4>(a.act, v[0], res);
 #pragma unroll
-              for (int r = 0; r < 4; ++r) res[r] *= v[1][r];
+              for (int r = 0; r < 4; ++r) res[r] *= v[NMAT - 1][r];
               store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
             } else {
-              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, v[0]);
-              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16, v[1]);
+#pragma unroll
+              for (int m = 0; m < NMAT; ++m) store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16 * m, v[m]);
             }
           }
 #pragma unroll
@@ -217,13 +221,13 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   wait_vmem<0>();
 }
 
-template <typename T, bool GATED>
+template <typename T, bool GATED, int NMAT>
 static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
-  constexpr int LDS = DS_WAVES * DS_RD * 2 * DS_REGION + 2 * (DS_WAVES - 1) * 2 * 256 * 4;
-  auto kern = decode_stream_kernel<T, GATED>;
+  constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT) * NMAT * DS_REGION + 2 * (DS_WAVES - 1) * NMAT * 256 * 4;
+  auto kern = decode_stream_kernel<T, GATED, NMAT>;
   static LdsAttrOnce lds_attr;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
-  int nblocks = a.R / (GATED ? 16 : 32);
+  int nblocks = a.R / (GATED ? 16 : 16 * NMAT);
   int grid = nblocks < num_cu ? nblocks : num_cu;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);
   return hipGetLastError();
@@ -243,10 +247,12 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
   if (hipError_t e = hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev)) return e;
   if (num_cu <= 0) num_cu = 256;
   StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act};
-  hipError_t e = launch_stream<T, true>(a1, num_cu, s);
+  hipError_t e = launch_stream<T, true, 2>(a1, num_cu, s);
   if (e != hipSuccess) return e;
   StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY};
-  return launch_stream<T, false>(a2, num_cu, s);
+  // 32-row blocks halve the L2 traffic for H, but only pay when they still occupy every CU
+  if (K / 32 >= num_cu) return launch_stream<T, false, 2>(a2, num_cu, s);
+  return launch_stream<T, false, 1>(a2, num_cu, s);
 }
 
 template hipError_t launch_decode_stream<f16>(const f16*, const f16*, const f16*, const f16*,

@@ -135,11 +135,11 @@ def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16)
 def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16, num_cu: int = 256) -> bool:
     """True when the skinny-M streaming kernels are the faster way to run the forward pass.
 
-    They hand out 16 rows of W_gate/W_up and 32 rows of W_down per workgroup and step; with fewer
-    than one such block per compute unit (hidden size below 32 * num_cu) the general path (gate/up
-    GEMM, down projection with a split reduction) is as fast or faster.
+    They hand out 16 rows of W_gate/W_up and 16 or 32 rows of W_down per workgroup and step; with
+    fewer than one such block per compute unit (hidden size below 16 * num_cu) the general path
+    (gate/up GEMM, down projection with a split reduction) is as fast or faster.
     """
-    return decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 32 * num_cu and K >= 32 * num_cu
+    return decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 32 * num_cu and K >= 16 * num_cu
 
 
 def decode_fwd(
