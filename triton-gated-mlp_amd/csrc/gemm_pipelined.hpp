@@ -19,16 +19,19 @@
 // B fragment (accumulator set b, column block j; G = NB * TN) with the step's TM A fragments.
 // Operands roll through registers instead of being double-buffered a whole step at a time:
 //   * A fragments: two banks of TM; during step s, group g fetches A fragment g of step s+1;
-//   * B fragments: a ring of 4; group g fetches the B fragment of group g+2.
+//   * B fragments: a ring of 4; group g fetches the B fragment of group g+LA (LA = 2 by default).
 // That is 2*TM + 4 fragments in flight (72 VGPRs for the 16x16x32 shape instead of 128), which is
 // what lets v_mfma_f32_16x16x32 be used with a 128x128 register tile: it moves a fifth fewer
 // register bytes per FLOP than 32x32x16 (4 accumulator floats per lane and instruction instead of
 // 16), and on MI355X, where these kernels run power-limited, that shows up as clock.
 //
 // A reduction tile's ring slot is retired at ONE barrier, placed in the tile's last step where the
-// rolling fetches stop addressing the tile: before group G-2.  After it, groups G-2 and G-1 fetch
+// rolling fetches stop addressing the tile: before group G-LA.  After it, the last LA groups fetch
 // the next tile's first B fragments and all of its first A fragments, and the global->LDS refill of
 // the freed slot starts, paced over the following MFMA slots.
+//
+// With a split-reduction epilogue (Epi::SPLIT) several workgroups share an output tile, each
+// reducing its own range of reduction tiles into a partial result.
 #pragma once
 #include "gemm_tiles.hpp"
 
