@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 3
+#define GMLP_ABI_VERSION 4
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -61,7 +61,13 @@ enum gmlp_status {
   GMLP_EHIP = -4    /* HIP runtime reported an error at launch */
 };
 
-enum gmlp_op { GMLP_OP_DECODE_FWD = 0, GMLP_OP_COLSUM = 1, GMLP_OP_LINEAR_FWD = 2, GMLP_OP_DX_BWD = 3 };
+enum gmlp_op {
+  GMLP_OP_DECODE_FWD = 0,
+  GMLP_OP_COLSUM = 1,
+  GMLP_OP_LINEAR_FWD = 2,
+  GMLP_OP_DX_BWD = 3,
+  GMLP_OP_GATEUP_FWD = 4
+};
 
 int gmlp_abi_version(void);
 const char* gmlp_last_error(void);
@@ -69,7 +75,8 @@ const char* gmlp_last_error(void);
 /*
  * Workspace bytes the caller must provide for `op` at the given problem size (0 if none), with
  * (M, K, N) as the entry point of that name takes them: GMLP_OP_COLSUM (M, 0, C),
- * GMLP_OP_LINEAR_FWD (M, R, C), GMLP_OP_DX_BWD (M, K, N), GMLP_OP_DECODE_FWD (M, K, N).
+ * GMLP_OP_LINEAR_FWD (M, R, C), GMLP_OP_DX_BWD (M, K, N), GMLP_OP_GATEUP_FWD (M, K, N),
+ * GMLP_OP_DECODE_FWD (M, K, N).
  */
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
 
@@ -81,11 +88,14 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
  * b_gate, b_up, g_save, u_save, mask_out may be NULL.  g_save/u_save [M,N] receive G and U
  * (activations kept for the backward pass).  mask_out [M,N] uint8 receives the keep mask.
  * Requires K % 8 == 0, N % 8 == 0, M >= 1.
+ * workspace (may be NULL): gmlp_workspace_bytes(GMLP_OP_GATEUP_FWD, M, K, N, dtype) bytes, used as
+ * in gmlp_linear_fwd (non-zero for short batches whose tiles would leave half the chip idle).
  */
 int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
                     const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
                     int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p,
-                    uint64_t seed, uint64_t offset, void* stream);
+                    uint64_t seed, uint64_t offset, void* workspace, size_t workspace_bytes,
+                    void* stream);
 
 /*
  * Linear layer forward: out[M,C] = a[M,R]·w[C,R]ᵀ + bias[C]   (bias may be NULL).

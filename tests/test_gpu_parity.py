@@ -156,6 +156,7 @@ def test_ragged_token_counts_on_the_pipelined_kernels(M, K, N, dtype, bias, p):
         (300, 1024, 4096, torch.bfloat16, True),
         (130, 4096, 14336, torch.float16, False),  # Llama-3-8B widths, short batch
         (40, 1024, 4160, torch.float16, False),  # 130 reduction tiles for dX do not divide by 16 splits
+        (100, 5120, 13824, torch.float16, True),  # Llama-2-13B widths: the gate/up GEMM splits as well
     ],
 )
 def test_short_batches_split_the_long_reductions(M, K, N, dtype, bias):
@@ -167,6 +168,8 @@ def test_short_batches_split_the_long_reductions(M, K, N, dtype, bias):
     code = _cabi.dtype_code(dtype)
     assert _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, M, N, K, code) > 0
     assert _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_DX_BWD, M, K, N, code) > 0
+    if N == 13824:
+        assert _cabi.lib().gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, M, K, N, code) > 0
     _run_module_case(Case(f"short_{M}x{K}x{N}", M, K, N, dtype, bias=bias, p=0.0, backward=True, seed=M + 1))
 
 

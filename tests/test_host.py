@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"libgmlp.so does not export {name}"
     assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
-    assert lib.gmlp_abi_version() == 3
+    assert lib.gmlp_abi_version() == 4
 
 
 def _buf(nbytes=4096):
@@ -50,15 +50,15 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 256, 2, 0, None) == -2
     # shape: K not a multiple of 8, M < 1
     assert lib.gmlp_linear_fwd(a, a, None, a, 8, 12, 8, 0, None, 0, None) == -2 and "multiple of 8" in err()
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0, 0.0, 0, 0, None) == -2
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 0, 8, 8, 0, 0, 0.0, 0, 0, None, 0, None) == -2
     # alignment
     assert lib.gmlp_linear_fwd(a + 2, a, None, a, 8, 8, 8, 0, None, 0, None) == -3 and "aligned" in err()
     # dropout probability outside [0, 1)
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, 1.0, 0, 0, None) == -1
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, -0.1, 0, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, 1.0, 0, 0, None, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 0, -0.1, 0, 0, None, 0, None) == -1
     assert lib.gmlp_dropout_mask(a, 8, 8, float("nan"), 0, 0, None) == -1
     # activation code outside the GMLP_ACT_* range
-    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 7, 0.0, 0, 0, None) == -1
+    assert lib.gmlp_gateup_fwd(a, a, a, None, None, a, None, None, None, 8, 8, 8, 0, 7, 0.0, 0, 0, None, 0, None) == -1
     assert "act" in err()
     assert lib.gmlp_gating_bwd(a, a, a, a, a, 8, 8, 0, -1, 0.0, 0, 0, None) == -1
     # decode limits
@@ -83,6 +83,11 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert n > 0 and n % (64 * 8192 * 4) == 0 and 2 <= n // (64 * 8192 * 4) <= 16
     n = lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DX_BWD, 300, 4096, 14336, 1)
     assert n > 0 and n % (300 * 4096 * 4) == 0
+    # gate/up: two accumulator sets per split; only when its 128 x 64 tiles leave the chip half idle
+    n = lib.gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, 64, 5120, 13824, 0)
+    assert n > 0 and n % (2 * 64 * 13824 * 4) == 0
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, 64, 8192, 28672, 0) == 0
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, 8192, 4096, 14336, 0) == 0
 
 
 def test_error_codes_map_to_python_exceptions():

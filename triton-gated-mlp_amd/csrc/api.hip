@@ -138,9 +138,10 @@ int pick_tile(int dtype, int64_t rows, int64_t cols, int64_t red, int bn_large, 
 // projection and input gradient of a short batch) leaves most of the chip idle and is bound by
 // streaming the weights; splitting the reduction fills two 128-tile workgroups per CU.  Each split
 // keeps at least 8 reduction tiles.
-int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_tiles) {
-  if (pick_tile(dtype, rows, cols, red, 256) != gmlp::TILE_MEDIUM_FULL) return 1;
-  const int64_t tiles = ((rows + 127) / 128) * ((cols + 127) / 128);
+int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_tiles, int bn_large = 256) {
+  if (pick_tile(dtype, rows, cols, red, bn_large) != gmlp::TILE_MEDIUM_FULL) return 1;
+  const int64_t bn = bn_large / 2;
+  const int64_t tiles = ((rows + 127) / 128) * ((cols + bn - 1) / bn);
   int64_t s = 2 * num_cu() / tiles;
   if (s > red_tiles / 8) s = red_tiles / 8;
   if (s > 16) s = 16;
@@ -151,8 +152,8 @@ int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_
   return (int)((red_tiles + per - 1) / per);
 }
 
-size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols) {
-  return splits > 1 ? (size_t)splits * rows * cols * sizeof(float) : 0;
+size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols, int accumulator_sets = 1) {
+  return splits > 1 ? (size_t)splits * accumulator_sets * rows * cols * sizeof(float) : 0;
 }
 
 }  // namespace
@@ -166,6 +167,9 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) 
   if (M < 1 || N < 1) return 0;
   if (op == GMLP_OP_COLSUM) return gmlp::colsum_workspace_bytes(M, N);
   if (K < 1) return 0;
+  // gmlp_gateup_fwd(M, K, N): two accumulator sets [M,N], reduction K
+  if (op == GMLP_OP_GATEUP_FWD)
+    return split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64, 128), M, N, 2);
   // gmlp_linear_fwd(M, R = K, C = N): out [M,N], reduction K
   if (op == GMLP_OP_LINEAR_FWD) return split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64), M, N);
   // gmlp_dx_bwd(M, K, N): out [M,K], reduction over two segments of N
@@ -176,7 +180,8 @@ size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) 
 int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const void* b_gate,
                     const void* b_up, void* h, void* g_save, void* u_save, uint8_t* mask_out,
                     int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p,
-                    uint64_t seed, uint64_t offset, void* stream) {
+                    uint64_t seed, uint64_t offset, void* workspace, size_t workspace_bytes,
+                    void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(x); GMLP_REQUIRE_PTR(w_gate); GMLP_REQUIRE_PTR(w_up); GMLP_REQUIRE_PTR(h);
   GMLP_REQUIRE_DTYPE(dtype);
@@ -189,17 +194,30 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   GMLP_REQUIRE_ALIGNED(x); GMLP_REQUIRE_ALIGNED(w_gate); GMLP_REQUIRE_ALIGNED(w_up);
   GMLP_REQUIRE_ALIGNED(b_gate); GMLP_REQUIRE_ALIGNED(b_up); GMLP_REQUIRE_ALIGNED(h);
   GMLP_REQUIRE_ALIGNED(g_save); GMLP_REQUIRE_ALIGNED(u_save); GMLP_REQUIRE_ALIGNED(mask_out);
+  GMLP_REQUIRE_ALIGNED(workspace);
 
   GemmArgs ga = {};
   ga.A[0] = x; ga.A[1] = x; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
   ga.nseg = 1; ga.group_m = 8;
   int tc = pick_tile(dtype, M, N, K, 128);
+  const int splits = pick_splits(dtype, M, N, K, (K + 63) / 64, 128);
+  const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, N, 2);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = by_dtype(dtype, [&](auto tag) {
+  hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
     typename EpiGateUp<T>::Args ea = {(T*)h, (T*)g_save, (T*)u_save, mask_out, (const T*)b_gate,
                                       (const T*)b_up, (int)N, act, d};
+    if constexpr (!std::is_same<T, float>::value) {
+      if (split) {
+        // per split: the gate partial sums [M,N], then the up partial sums [M,N]
+        ga.splits = splits;
+        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)2 * M * N, (size_t)M * N, (int)N};
+        if (hipError_t err = launch_gateup_split<T>(ga, pa, s)) return err;
+        return launch_splitk_reduce<T, EpiGateUp<T>>((const float*)workspace, splits, (size_t)2 * M * N,
+                                                     (size_t)M * N, ea, M, N, s);
+      }
+    }
     return launch_gateup<T>(tc, ga, ea, s);
   });
   return hip_result(__func__, e);
@@ -229,9 +247,10 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
     if constexpr (!std::is_same<T, float>::value) {
       if (split) {
         ga.splits = splits;
-        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * C, (int)C};
+        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * C, 0, (int)C};
         if (hipError_t err = launch_linear_split<T>(ga, pa, s)) return err;
-        return launch_splitk_reduce<T>((const float*)workspace, splits, (size_t)M * C, (const T*)bias, (T*)out, M, C, s);
+        typename EpiStore<T>::Args ea = {(T*)out, (const T*)bias, (int)C};
+        return launch_splitk_reduce<T, EpiStore<T>>((const float*)workspace, splits, (size_t)M * C, 0, ea, M, C, s);
       }
     }
     typename EpiStore<T>::Args ea = {(T*)out, (const T*)bias, (int)C};
@@ -320,9 +339,10 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
     if constexpr (!std::is_same<T, float>::value) {
       if (split) {
         ga.splits = splits;
-        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * K, (int)K};
+        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * K, 0, (int)K};
         if (hipError_t err = launch_dx_split<T>(ga, pa, s)) return err;
-        return launch_splitk_reduce<T>((const float*)workspace, splits, (size_t)M * K, (const T*)nullptr, (T*)dx, M, K, s);
+        typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};
+        return launch_splitk_reduce<T, EpiStore<T>>((const float*)workspace, splits, (size_t)M * K, 0, ea, M, K, s);
       }
     }
     typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};

@@ -38,43 +38,52 @@ template hipError_t launch_gating_bwd<float>(const float*, const float*, const f
                                              float*, int64_t, int64_t, int, const DropoutParams&,
                                              hipStream_t);
 
-// Second stage of a split reduction: adds the partial results up in split order (deterministic).
-template <typename T>
+// Second stage of a split reduction: adds the partial results up in split order (deterministic)
+// and hands 8 consecutive columns of one row to the epilogue the unsplit GEMM would have run.
+template <typename T, typename Epi>
 __global__ void __launch_bounds__(256)
-    splitk_reduce_kernel(const float* __restrict__ ws, int splits, size_t stride,
-                         const T* __restrict__ bias, T* __restrict__ out, size_t n8, int N) {
+    splitk_reduce_kernel(const float* __restrict__ ws, int splits, size_t split_stride, size_t acc_stride,
+                         typename Epi::Args ea, size_t n8, int N) {
   size_t step = (size_t)gridDim.x * blockDim.x;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += step) {
     size_t e = i * 8;
-    float v[8];
+    alignas(16) float v0[8], v1[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) v[r] = 0.f;
+    for (int r = 0; r < 8; ++r) v0[r] = v1[r] = 0.f;
     for (int s = 0; s < splits; ++s) {
-      const float* p = ws + (size_t)s * stride + e;
+      const float* p = ws + (size_t)s * split_stride + e;
       f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) { v[r] += a[r]; v[4 + r] += b[r]; }
+      for (int r = 0; r < 4; ++r) { v0[r] += a[r]; v0[4 + r] += b[r]; }
+      if (acc_stride) {
+        f32x4 c = *(const f32x4*)(p + acc_stride), d = *(const f32x4*)(p + acc_stride + 4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { v1[r] += c[r]; v1[4 + r] += d[r]; }
+      }
     }
-    if (bias) add_w<T, 8>(bias + (e % (size_t)N), v);
-    store_w<T, 8>(out + e, v);
+    Epi::template apply<8>(ea, (int)(e / (size_t)N), (int)(e % (size_t)N), v0, v1);
   }
 }
 
-template <typename T>
-hipError_t launch_splitk_reduce(const float* ws, int splits, size_t stride, const T* bias, T* out,
-                                int64_t M, int64_t N, hipStream_t s) {
+template <typename T, typename Epi>
+hipError_t launch_splitk_reduce(const float* ws, int splits, size_t split_stride, size_t acc_stride,
+                                const typename Epi::Args& ea, int64_t M, int64_t N, hipStream_t s) {
   size_t n8 = (size_t)M * N / 8;
   if (n8 == 0) return hipSuccess;
   size_t blocks = (n8 + 255) / 256;
   if (blocks > 256 * 8) blocks = 256 * 8;
-  hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, ws, splits, stride,
-                     bias, out, n8, (int)N);
+  hipLaunchKernelGGL((splitk_reduce_kernel<T, Epi>), dim3((unsigned)blocks), dim3(256), 0, s, ws, splits,
+                     split_stride, acc_stride, ea, n8, (int)N);
   return hipGetLastError();
 }
-template hipError_t launch_splitk_reduce<f16>(const float*, int, size_t, const f16*, f16*, int64_t,
-                                              int64_t, hipStream_t);
-template hipError_t launch_splitk_reduce<bf16>(const float*, int, size_t, const bf16*, bf16*, int64_t,
-                                               int64_t, hipStream_t);
+#define GMLP_REDUCE_INST(T, EPI)                                                                    \
+  template hipError_t launch_splitk_reduce<T, EPI<T>>(const float*, int, size_t, size_t,            \
+                                                      const EPI<T>::Args&, int64_t, int64_t, hipStream_t);
+GMLP_REDUCE_INST(f16, EpiStore)
+GMLP_REDUCE_INST(bf16, EpiStore)
+GMLP_REDUCE_INST(f16, EpiGateUp)
+GMLP_REDUCE_INST(bf16, EpiGateUp)
+#undef GMLP_REDUCE_INST
 
 // Column sums in two fixed-order stages: COLSUM_SPLITS row ranges -> fp32 partials -> total.
 // Up to COLSUM_GROUP_MAX arrays with the same number of rows share the two launches (the bias

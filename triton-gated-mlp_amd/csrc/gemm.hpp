@@ -310,12 +310,14 @@ struct EpiStore {
 };
 
 // Split reduction: workgroup `split` of an output tile stores its fp32 partial sums to
-// ws[split][m][n]; splitk_reduce (aux.hip) adds the partials up and applies EpiStore.
+// ws[split][acc][m][n] (acc: accumulator set, for NB == 2); splitk_reduce (aux.hip) adds the
+// partials up and applies the real epilogue.
 template <typename T>
 struct EpiPartial {
   struct Args {
     float* ws;
     size_t split_stride;  // elements between the partial results of consecutive splits
+    size_t acc_stride;    // elements between the two accumulator sets of one split (0: one set)
     int ldc;
   };
   static constexpr int PREFETCH_DEPTH = 0;
@@ -326,11 +328,15 @@ struct EpiPartial {
   template <int W>
   static __device__ __forceinline__ void prefetch(const Args&, int, int, Prefetch<W>&) {}
   template <int W, int ACT>
-  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float*,
+  static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v0, float* v1,
                                                const Prefetch<W>&) {
     float* p = a.ws + (size_t)m * a.ldc + n;
 #pragma unroll
-    for (int q = 0; q < W / 4; ++q) *(f32x4*)(p + 4 * q) = *(const f32x4*)(v + 4 * q);
+    for (int q = 0; q < W / 4; ++q) *(f32x4*)(p + 4 * q) = *(const f32x4*)(v0 + 4 * q);
+    if (a.acc_stride) {
+#pragma unroll
+      for (int q = 0; q < W / 4; ++q) *(f32x4*)(p + a.acc_stride + 4 * q) = *(const f32x4*)(v1 + 4 * q);
+    }
   }
 };
 

@@ -34,6 +34,10 @@ hipError_t launch_gateup<DT>(int tile_class, const GemmArgs& ga, const EpiGateUp
                              hipStream_t s) {
   GMLP_DISPATCH(false, false, 2, EpiGateUp, 128, 64)
 }
+template <>
+hipError_t launch_gateup_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
+  return launch_gemm_pipelined<DT, 128, 64, GMLP_MI, 2, 2, false, false, 2, EpiPartial<DT>>(ga, ea, s);
+}
 #elif GMLP_KIND == 1
 template <>
 hipError_t launch_linear<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>::Args& ea,

@@ -52,6 +52,8 @@ template <typename T>
 hipError_t launch_linear_split(const GemmArgs& ga, const typename EpiPartial<T>::Args& ea, hipStream_t s);
 template <typename T>
 hipError_t launch_dx_split(const GemmArgs& ga, const typename EpiPartial<T>::Args& ea, hipStream_t s);
+template <typename T>
+hipError_t launch_gateup_split(const GemmArgs& ga, const typename EpiPartial<T>::Args& ea, hipStream_t s);
 
 // decode.hip
 template <typename T>
@@ -70,10 +72,11 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
 template <typename T>
 hipError_t launch_gating_bwd(const T* dh, const T* g, const T* u, T* dg, T* du, int64_t M, int64_t N,
                              int act, const DropoutParams& d, hipStream_t s);
-// out[m,n] = sum_s ws[s*stride + m*N + n] (+ bias[n]): second stage of a split reduction
-template <typename T>
-hipError_t launch_splitk_reduce(const float* ws, int splits, size_t stride, const T* bias, T* out,
-                                int64_t M, int64_t N, hipStream_t s);
+// Second stage of a split reduction: Epi (EpiStore or EpiGateUp) applied to
+// sum_s ws[s*split_stride (+ acc_stride) + m*N + n].
+template <typename T, typename Epi>
+hipError_t launch_splitk_reduce(const float* ws, int splits, size_t split_stride, size_t acc_stride,
+                                const typename Epi::Args& ea, int64_t M, int64_t N, hipStream_t s);
 constexpr int COLSUM_GROUP_MAX = 3;
 template <typename T>
 struct ColsumGroup {

@@ -15,8 +15,8 @@ import torch
 from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
-GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD = 0, 1, 2, 3
-ABI_VERSION = 3
+GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD, GMLP_OP_GATEUP_FWD = 0, 1, 2, 3, 4
+ABI_VERSION = 4
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
 # tables (src/triton_gated_mlp/gated_mlp.py:17-37).
@@ -43,7 +43,10 @@ _SIGNATURES = {
     "gmlp_abi_version": (_int, []),
     "gmlp_last_error": (ctypes.c_char_p, []),
     "gmlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
-    "gmlp_gateup_fwd": (_int, [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_gateup_fwd": (
+        _int,
+        [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr, ctypes.c_size_t, _c_ptr],
+    ),
     "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
     "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
     "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),

@@ -70,11 +70,13 @@ def gateup_fwd(
     mask = torch.empty((M, N), dtype=torch.uint8, device=dev) if return_mask else None
     if M > 0:
         with torch.cuda.device(dev):
+            ws = _cabi.workspace(_cabi.GMLP_OP_GATEUP_FWD, M, K, N, code, dev)
             _cabi.check(
                 _cabi.lib().gmlp_gateup_fwd(
                     _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(b_gate), _cabi.ptr(b_up),
                     _cabi.ptr(h), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(mask),
-                    M, K, N, code, act, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                    M, K, N, code, act, float(dropout_p), int(seed), int(offset),
+                    _cabi.ptr(ws), 0 if ws is None else ws.numel(), _cabi.stream_ptr(dev),
                 )
             )
     return HiddenStates(h, g, u, mask)
@@ -135,11 +137,15 @@ def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16)
 def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16, num_cu: int = 256) -> bool:
     """True when the skinny-M streaming kernels are the faster way to run the forward pass.
 
-    They hand out 16 rows of W_gate/W_up and 16 or 32 rows of W_down per workgroup and step; with
-    fewer than one such block per compute unit (hidden size below 16 * num_cu) the general path
-    (gate/up GEMM, down projection with a split reduction) is as fast or faster.
+    They hand out 16 rows of W_gate/W_up and 16 or 32 rows of W_down per workgroup and step.  With
+    at least one 32-row block per compute unit (both widths >= 32 * num_cu) they win for every
+    M <= 16; down to half that hidden size they still win for M <= 8; below, the general path
+    (GEMMs with split reductions) is as fast or faster.  Measured on MI355X at the widths of
+    Llama-2-7B/13B, Llama-3-8B and Llama-3-70B.
     """
-    return decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 32 * num_cu and K >= 16 * num_cu
+    if not (decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 32 * num_cu):
+        return False
+    return K >= 32 * num_cu or (M <= 8 and K >= 16 * num_cu)
 
 
 def decode_fwd(
