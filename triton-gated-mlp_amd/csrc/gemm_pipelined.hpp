@@ -308,7 +308,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // are dropped when it comes to storing.
   constexpr int ITEMS = MI * WTN / 8 / 64;  // items per lane and slab
   constexpr int NITEMS = TM * ITEMS;
-  constexpr int PD = Epi::PREFETCH_DEPTH < NITEMS ? Epi::PREFETCH_DEPTH : NITEMS;
+  // (the 32x32x16 instance has fewer registers to spare; the depth hardly matters, 4 = 8 = 12 measured)
+  constexpr int PD_WANTED = MI == 32 && Epi::PREFETCH_DEPTH > 4 ? 4 : Epi::PREFETCH_DEPTH;
+  constexpr int PD = PD_WANTED < NITEMS ? PD_WANTED : NITEMS;
   static_assert(MI * WTN / 8 % 64 == 0, "slab items must divide over the lanes");
   auto item_pos = [&](int q, int& row, int& m, int& n, int& cg) __attribute__((always_inline)) {
     int i = q / ITEMS, item = (q % ITEMS) * 64 + lane;
