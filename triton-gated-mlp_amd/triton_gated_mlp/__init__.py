@@ -1,6 +1,6 @@
 """MI355X-native fused gated MLP with the import surface of matteobonotto/triton-gated-mlp."""
 
-from . import gated_mlp, utils  # noqa: F401
+from . import const, gated_mlp, utils  # noqa: F401
 from .gated_mlp import (  # noqa: F401
     ACT_FWD,
     EagerGatedMLP,
