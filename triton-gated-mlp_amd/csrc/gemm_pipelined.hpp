@@ -19,7 +19,7 @@
 // B fragment (accumulator set b, column block j; G = NB * TN) with the step's TM A fragments.
 // Operands roll through registers instead of being double-buffered a whole step at a time:
 //   * A fragments: two banks of TM; during step s, group g fetches A fragment g of step s+1;
-//   * B fragments: a ring of 4; group g fetches the B fragment of group g+LA (LA = 2 by default).
+//   * B fragments: a ring of 4; group g fetches the B fragment of group g+LA (LA = 3 by default).
 // That is 2*TM + 4 fragments in flight (72 VGPRs for the 16x16x32 shape instead of 128), which is
 // what lets v_mfma_f32_16x16x32 be used with a 128x128 register tile: it moves a fifth fewer
 // register bytes per FLOP than 32x32x16 (4 accumulator floats per lane and instruction instead of
@@ -41,7 +41,7 @@ namespace gmlp {
 #define GMLP_LOAD_CYCLES 64  // one global->LDS load per this many MFMA cycles
 #endif
 #ifndef GMLP_B_LOOKAHEAD
-#define GMLP_B_LOOKAHEAD 2  // MFMA groups between the fetch of a B fragment and its use (2 or 3)
+#define GMLP_B_LOOKAHEAD 3  // MFMA groups between the fetch of a B fragment and its use (2 or 3)
 #endif
 
 template <int MI>
