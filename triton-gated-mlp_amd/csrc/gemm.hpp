@@ -255,12 +255,15 @@ struct PackW<T, 4> { typedef typename Traits<T>::vec4 type; };
 template <typename T>
 struct PackW<T, 8> { typedef typename Traits<T>::vec8 type; };
 
-template <typename T, int W>
+// STREAM: non-temporal store, for results nobody reads soon (layer outputs, gradients handed to
+// other layers or to the optimizer): they then do not push operand panels out of the caches.
+template <typename T, int W, bool STREAM = false>
 __device__ __forceinline__ void store_w(T* p, const float* v) {
   typename PackW<T, W>::type o;
 #pragma unroll
   for (int r = 0; r < W; ++r) o[r] = Traits<T>::from_f32(v[r]);
-  *(typename PackW<T, W>::type*)p = o;
+  if (STREAM) __builtin_nontemporal_store(o, (typename PackW<T, W>::type*)p);
+  else *(typename PackW<T, W>::type*)p = o;
 }
 template <typename T, int W>
 __device__ __forceinline__ void load_w(const T* p, float* v) {
@@ -292,7 +295,7 @@ struct EpiStore {
   template <int W>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* v, float*) {
     if (a.bias) add_w<T, W>(a.bias + n, v);
-    store_w<T, W>(a.out + (size_t)m * a.ldc + n, v);
+    store_w<T, W, true>(a.out + (size_t)m * a.ldc + n, v);
   }
   // Nothing worth fetching ahead of time (see EpiDh), no activation to specialise on.
   static constexpr int PREFETCH_DEPTH = 0;
