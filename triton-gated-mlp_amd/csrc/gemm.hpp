@@ -426,8 +426,8 @@ __device__ __forceinline__ void gating_bwd_core(int act, const DropoutParams& dr
     duv[r] = dh[r] * av[r];
     dgv[r] = dh[r] * Traits<T>::to_f32(up[r]) * dv[r];
   }
-  store_w<T, W>(dg + e, dgv);
-  store_w<T, W>(du + e, duv);
+  store_w<T, W, true>(dg + e, dgv);  // 2*M*N elements: more than the caches keep for the next kernels
+  store_w<T, W, true>(du + e, duv);
 }
 template <typename T, int W>
 __device__ __forceinline__ void gating_bwd_w(int act, const DropoutParams& drop, size_t e,
@@ -462,8 +462,8 @@ struct EpiDh {
   static __device__ __forceinline__ void prefetch(const Args& a, int m, int n, Prefetch<W>& p) {
     typedef typename PackW<T, W>::type pack;
     size_t e = (size_t)m * a.ldc + n;
-    p.g = *(const pack*)(a.g + e);
-    p.u = *(const pack*)(a.u + e);
+    p.g = __builtin_nontemporal_load((const pack*)(a.g + e));  // read once
+    p.u = __builtin_nontemporal_load((const pack*)(a.u + e));
   }
   static constexpr bool HAS_ACT = true;
   static constexpr bool SPLIT = false;
