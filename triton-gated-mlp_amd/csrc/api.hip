@@ -86,6 +86,10 @@ int hip_result(const char* fn, hipError_t e) {
   return fail(GMLP_EHIP, "%s: HIP error %d (%s)", fn, (int)e, hipGetErrorString(e));
 }
 
+// Scheduling groups of 8 tile-rows when the A operand (rows x red) is the smaller one, of 8
+// tile-columns (negative) when B (cols x red, `sets` of them) is: see tile_of_grouped.
+int pick_group(int64_t rows, int64_t cols, int sets = 1) { return sets * cols < rows ? -8 : 8; }
+
 // Compute units of the current device.
 int num_cu() {
   static int cached[64] = {};
@@ -199,7 +203,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   GemmArgs ga = {};
   ga.A[0] = x; ga.A[1] = x; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
-  ga.nseg = 1; ga.group_m = 8;
+  ga.nseg = 1; ga.group_m = pick_group(M, N, 2);
   int tc = pick_tile(dtype, M, N, K, 128);
   const int splits = pick_splits(dtype, M, N, K, (K + 63) / 64, 128);
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, N, 2);
@@ -237,7 +241,7 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   GemmArgs ga = {};
   ga.A[0] = a; ga.A[1] = a; ga.B[0] = w; ga.B[1] = w;
   ga.M = (int)M; ga.N = (int)C; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
-  ga.nseg = 1; ga.group_m = 8;
+  ga.nseg = 1; ga.group_m = pick_group(M, C);
   int tc = pick_tile(dtype, M, C, R, 256);
   const int splits = pick_splits(dtype, M, C, R, (R + 63) / 64);
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, C);
@@ -279,7 +283,7 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   GemmArgs ga = {};
   ga.A[0] = dy; ga.A[1] = dy; ga.B[0] = w_down; ga.B[1] = w_down;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
-  ga.nseg = 1; ga.group_m = 8;
+  ga.nseg = 1; ga.group_m = pick_group(M, N);
   int tc = pick_tile(dtype, M, N, K, 256);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
@@ -329,7 +333,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   GemmArgs ga = {};
   ga.A[0] = dg; ga.A[1] = du; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
-  ga.nseg = 2; ga.group_m = 8;
+  ga.nseg = 2; ga.group_m = pick_group(M, K);
   int tc = pick_tile(dtype, M, K, N, 256);
   const int splits = pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64));
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, K);
@@ -365,7 +369,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   GemmArgs ga = {};
   ga.A[0] = lhs; ga.A[1] = lhs; ga.B[0] = rhs; ga.B[1] = rhs;
   ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
-  ga.nseg = 1; ga.group_m = 8;
+  ga.nseg = 1; ga.group_m = pick_group(R, C);
   int tc = pick_tile(dtype, R, C, Mred, 256, true);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
@@ -411,7 +415,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     ga = GemmArgs{};
     ga.A[0] = lhs[i]; ga.A[1] = lhs[i]; ga.B[0] = rhs[i]; ga.B[1] = rhs[i];
     ga.M = (int)R[i]; ga.N = (int)C[i]; ga.K = (int)Mred; ga.lda = (int)R[i]; ga.ldb = (int)C[i];
-    ga.nseg = 1; ga.group_m = 8;
+    ga.nseg = 1; ga.group_m = pick_group(R[i], C[i]);
   };
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;

@@ -25,7 +25,7 @@ struct GemmArgs {
   int M, N, K;       // output rows, output cols, reduction length of one segment
   int lda, ldb;      // leading dimensions (elements)
   int nseg;          // number of reduction segments (1 or 2)
-  int group_m;       // tile-rows per scheduling group
+  int group_m;       // tile-rows per scheduling group; negative: -group_m tile-COLUMNS per group
   int splits;        // pipelined kernel with a split-reduction epilogue only: number of workgroups
                      // that share one output tile, each reducing a contiguous range of 64-wide
                      // reduction tiles into a partial result of its own (0 or 1: no split)
@@ -50,9 +50,21 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int gro
   tm = first_m + r % gsz;
   tn = r / gsz;
 }
+// group > 0: groups of `group` tile-rows, walked column by column: an XCD's successive rounds of
+// workgroups keep their A panels and move on to new B panels.  group < 0: the same with rows and
+// columns exchanged (B panels kept).  The kept operand should be the smaller one: it is the one
+// the memory-side cache can still hold when the next round asks for it again.
+__device__ __forceinline__ void tile_of_grouped(int t, int tiles_m, int tiles_n, int group, int& tm, int& tn) {
+  const bool by_columns = group < 0;
+  int major, minor;
+  tile_of(t, by_columns ? tiles_n : tiles_m, by_columns ? tiles_m : tiles_n, by_columns ? -group : group,
+          major, minor);
+  tm = by_columns ? minor : major;
+  tn = by_columns ? major : minor;
+}
 __device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tiles_n, int group_m,
                                          int& tm, int& tn) {
-  tile_of(xcd_contiguous(pid, nwg), tiles_m, tiles_n, group_m, tm, tn);
+  tile_of_grouped(xcd_contiguous(pid, nwg), tiles_m, tiles_n, group_m, tm, tn);
 }
 
 template <int BK>

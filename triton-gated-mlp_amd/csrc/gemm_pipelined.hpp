@@ -119,8 +119,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const int u = xcd_contiguous(pid, nwg);
   const int split = Epi::SPLIT ? u / ntiles : 0;
   int tm_i, tn_i;
-  tile_of(u - split * ntiles, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
-  const int m0 = tm_i * BM, n0 = tn_i * BN;
+  tile_of_grouped(u - split * ntiles, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  // workgroup-uniform by construction; say so, the tile origins feed scalar operands
+  const int m0 = __builtin_amdgcn_readfirstlane(tm_i) * BM, n0 = __builtin_amdgcn_readfirstlane(tn_i) * BN;
   typename Epi::Args ea = ea_in;
   if constexpr (Epi::SPLIT) ea.ws += (size_t)split * ea.split_stride;
 
