@@ -620,3 +620,32 @@ def test_forward_backward_under_hip_graph_replay():
         torch.cuda.synchronize(dev)
         for name, got, ref in zip(["Y", "dX"] + [n for n, _ in mlp.named_parameters()], outs, eager):
             assert torch.equal(got, ref), f"replay {rep}: {name} differs from the eager step"
+
+
+@pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])
+def test_autocast_with_fp32_master_weights(amp_dtype):
+    """Mixed-precision training: fp32 parameters, torch.autocast picks the kernel dtype; gradients
+    come back in fp32 and match the oracle evaluated on the rounded operands."""
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    c = Case("amp", 384, 256, 640, amp_dtype, bias=True, backward=True, seed=41)
+    t = make_inputs(c)  # values already representable in amp_dtype
+    mlp = FusedGatedMLP(c.K, c.N, bias=True).to(dev).float()
+    with torch.no_grad():
+        for name, key in (("gate_proj", "gate"), ("up_proj", "up"), ("down_proj", "down")):
+            getattr(mlp, name).weight.copy_(t[f"W_{key}"].float())
+            getattr(mlp, name).bias.copy_(t[f"b_{key}"].float())
+    x = t["x"].float().to(dev).requires_grad_(True)
+    with torch.autocast("cuda", dtype=amp_dtype):
+        y = mlp(x)
+    assert y.dtype == amp_dtype
+    params = [x] + list(mlp.parameters())
+    grads = torch.autograd.grad(y, params, grad_outputs=t["dY"].to(dev))
+    assert all(g.dtype == torch.float32 for g in grads), "master-weight gradients must stay fp32"
+    o = _oracle_inputs(t)
+    ref = oracle.backward(o["x"], o["W_gate"], o["b_gate"], o["W_up"], o["b_up"], o["W_down"], o["b_down"], o["dY"])
+    _close("Y", y, ref["Y"])
+    names = ["dX", "dW_gate", "db_gate", "dW_up", "db_up", "dW_down", "db_down"]
+    for n, g in zip(names, grads):
+        _close(n, g, ref[n], atol=ATOL * max(1.0, ref[n].abs().mean().item()))

@@ -206,6 +206,9 @@ class FusedGatedMLP(_GatedMLPBase):
     torch's default CPU generator (so `torch.manual_seed` makes runs repeatable).  The seed and
     offset of the last training forward are kept in `last_dropout_state`.
 
+    Under `torch.autocast("cuda")` the module casts its input and parameters to the autocast dtype
+    for the kernels (fp32 master weights keep fp32 gradients), as nn.Linear does.
+
     `recompute_activations = True` selects the memory-lean backward: only x is kept from the forward
     pass and G, U, H are recomputed (one more gate/up GEMM) instead of holding 3*M*N elements.
     """
@@ -231,6 +234,23 @@ class FusedGatedMLP(_GatedMLPBase):
         x2 = x.reshape(-1, x.shape[-1])
         p = float(self.dropout.p) if self.training else 0.0
         gate, up, down = self.gate_proj, self.up_proj, self.down_proj
+        if x2.is_cuda and torch.is_autocast_enabled("cuda"):
+            # Mixed precision as nn.Linear does it under torch.autocast: activations and (master)
+            # weights are cast to the autocast dtype for the kernels; autograd casts the gradients back.
+            with torch.autocast("cuda", enabled=False):
+                return self._forward_cast(x2, torch.get_autocast_dtype("cuda"), p).reshape(*lead, self.hidden_size)
+        return self._forward_2d(
+            x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p
+        ).reshape(*lead, self.hidden_size)
+
+    def _forward_cast(self, x2: Tensor, dtype: torch.dtype, p: float) -> Tensor:
+        cast = lambda t: None if t is None else t.to(dtype)
+        g, u, d = self.gate_proj, self.up_proj, self.down_proj
+        return self._forward_2d(
+            cast(x2), cast(g.weight), cast(g.bias), cast(u.weight), cast(u.bias), cast(d.weight), cast(d.bias), p
+        )
+
+    def _forward_2d(self, x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p: float) -> Tensor:
         M, K = x2.shape
         inference = not torch.is_grad_enabled() or not (
             x2.requires_grad or any(q.requires_grad for q in self.parameters())
@@ -238,13 +258,8 @@ class FusedGatedMLP(_GatedMLPBase):
         if inference and p == 0.0 and x2.is_cuda and _fwd.decode_preferred(
             M, K, self.intermediate_size, x2.dtype, torch.cuda.get_device_properties(x2.device).multi_processor_count
         ):
-            y = _fwd.decode_fwd(
-                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, self.act_fn
-            )
-        else:
-            seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
-            y = FusedGatedMLPFullFunction.apply(
-                x2, gate.weight, gate.bias, up.weight, up.bias, down.weight, down.bias, p, seed, offset,
-                self.recompute_activations, self.act_fn,
-            )
-        return y.reshape(*lead, self.hidden_size)
+            return _fwd.decode_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, self.act_fn)
+        seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
+        return FusedGatedMLPFullFunction.apply(
+            x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p, seed, offset, self.recompute_activations, self.act_fn
+        )
