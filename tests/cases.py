@@ -1,4 +1,4 @@
-"""Seeded inputs of the BASELINE configurations, generated on the CPU so that the HIP path and the
+"""Seeded inputs of the five benchmark configurations, generated on the CPU so that the HIP path and the
 oracle see bit-identical tensors."""
 
 from __future__ import annotations
