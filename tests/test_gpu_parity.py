@@ -250,6 +250,38 @@ def test_other_activations_operator_level(act):
     _close("dW_gate", dWg, hb["dG"].T @ o["x"], atol=ATOL * max(1.0, (hb["dG"].T @ o["x"]).abs().mean().item()))
 
 
+def test_device_activation_functions_against_float64_closed_forms():
+    """The kernels evaluate erf and tanh through short fp32 approximations; this pins them far below
+    the storage tolerance.  gating_bwd in float32 with dH = U = 1 returns act(G) as dU and act'(G) as
+    dG, compared with scipy / numpy in float64 on a dense grid that includes both tails and 0."""
+    from scipy.special import erf, expit
+
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    x32 = torch.linspace(-12.0, 12.0, 64 * 4096, dtype=torch.float32).reshape(64, 4096).clone()
+    x32[0, :2] = torch.tensor([0.0, -0.0])
+    x = x32.double().numpy()
+    cdf, pdf = 0.5 * (1.0 + erf(x / np.sqrt(2.0))), np.exp(-0.5 * x * x) / np.sqrt(2.0 * np.pi)
+    closed = {
+        "silu": (x * expit(x), expit(x) * (1.0 + x * (1.0 - expit(x)))),
+        "gelu": (x * cdf, cdf + x * pdf),
+        "sigmoid": (expit(x), expit(x) * (1.0 - expit(x))),
+        "tanh": (np.tanh(x), 1.0 - np.tanh(x) ** 2),
+    }
+    one = torch.ones_like(x32).to(dev)
+    for act, (f, df) in closed.items():
+        dg, du = ops_bwd.gating_bwd(one, x32.to(dev), one, 0.0, 0, 0, act)
+        err_f = np.abs(du.cpu().double().numpy() - f).max()
+        err_d = np.abs(dg.cpu().double().numpy() - df).max()
+        assert err_f < 2e-6 and err_d < 2e-6, (act, err_f, err_d)  # |x| <= 12: a few fp32 ulps of the value
+    # tanh keeps its relative accuracy through 0 (no 1 - e^{-2x} cancellation)
+    tiny = torch.logspace(-6, -1, 4096, dtype=torch.float32).reshape(1, -1)
+    _, du = ops_bwd.gating_bwd(torch.ones_like(tiny).to(dev), tiny.to(dev), torch.ones_like(tiny).to(dev), 0.0, 0, 0, "tanh")
+    rel = np.abs(du.cpu().double().numpy() / np.tanh(tiny.double().numpy()) - 1.0).max()
+    assert rel < 1e-6, rel
+
+
 def test_three_dimensional_input_matches_flattened():
     """[B, S, K] input gives the 2-D result on x.view(-1, K) (tests/test_gated_mlp_bwd.py:37-45)."""
     from triton_gated_mlp import FusedGatedMLP

@@ -69,6 +69,36 @@ __device__ __forceinline__ float silu_grad_f32(float x) {
   return s * (1.0f + x * (1.0f - s));
 }
 
+// Phi(x) = (1 + erf(x/sqrt 2))/2 through Abramowitz & Stegun 7.1.26, erfc(z) = poly(t) e^{-z^2} with
+// t = 1/(1 + p z) for z >= 0 (|error| <= 1.5e-7 on erf, so <= 3e-7 on Phi with fp32 rounding: three
+// orders below fp16/bf16 resolution).  One exp and one reciprocal per value instead of libm's
+// two-branch erff, and e^{-x^2/2} is shared with the normal density the derivative needs.  The
+// lower tail comes out as a product rather than as 1 + erf, so it does not cancel.
+struct NormalCdf {
+  float cdf, e;  // Phi(x), e^{-x^2/2}
+};
+__device__ __forceinline__ NormalCdf normal_cdf_f32(float x) {
+  const float ax = fabsf(x);
+  const float t = 1.0f / (1.0f + 0.23164189f * ax);  // p / sqrt 2, p = 0.3275911
+  const float e = __expf(-0.5f * x * x);
+  float poly = 1.061405429f;
+  poly = poly * t - 1.453152027f;
+  poly = poly * t + 1.421413741f;
+  poly = poly * t - 0.284496736f;
+  poly = poly * t + 0.254829592f;
+  const float q = 0.5f * poly * t * e;
+  return {x < 0.f ? q : 1.0f - q, e};
+}
+// tanh(x) = sign(x) (1 - e)/(1 + e), e = e^{-2|x|}; below 1/4 the odd series to x^7 (next term
+// 62/2835 x^9 < 2e-7 relative) replaces the cancelling 1 - e.  Relative error < 5e-7.
+__device__ __forceinline__ float tanh_f32(float x) {
+  const float ax = fabsf(x), x2 = x * x;
+  const float e = __expf(-2.0f * ax);
+  const float big = (1.0f - e) / (1.0f + e);
+  const float small = ax * (1.0f + x2 * (-0.33333333f + x2 * (0.13333333f - x2 * 0.053968254f)));
+  return copysignf(ax < 0.25f ? small : big, x);
+}
+
 // Gate activations.  The codes are the GMLP_ACT_* values of the C interface; the functions are the
 // ones the reference's eager module offers for hidden_act (ACT2CLS / ACT_FWD,
 // src/triton_gated_mlp/gated_mlp.py:17-37) with torch's default parameters: exact (erf) GELU,
@@ -99,7 +129,7 @@ __device__ __forceinline__ void act_fwd_w(int act, const float* x, float* y) {
       break;
     case ACT_GELU:
 #pragma unroll
-      for (int r = 0; r < W; ++r) y[r] = 0.5f * x[r] * (1.0f + erff(x[r] * 0.70710678118654752f));
+      for (int r = 0; r < W; ++r) y[r] = x[r] * normal_cdf_f32(x[r]).cdf;
       break;
     case ACT_RELU:
 #pragma unroll
@@ -115,7 +145,7 @@ __device__ __forceinline__ void act_fwd_w(int act, const float* x, float* y) {
       break;
     case ACT_TANH:
 #pragma unroll
-      for (int r = 0; r < W; ++r) y[r] = tanhf(x[r]);
+      for (int r = 0; r < W; ++r) y[r] = tanh_f32(x[r]);
       break;
     default:
 #pragma unroll
@@ -139,10 +169,9 @@ __device__ __forceinline__ void act_fwd_grad_w(int act, const float* x, float* y
     case ACT_GELU:
 #pragma unroll
       for (int r = 0; r < W; ++r) {
-        float cdf = 0.5f * (1.0f + erff(x[r] * 0.70710678118654752f));
-        float pdf = 0.39894228040143268f * __expf(-0.5f * x[r] * x[r]);
-        y[r] = x[r] * cdf;
-        d[r] = cdf + x[r] * pdf;
+        NormalCdf n = normal_cdf_f32(x[r]);
+        y[r] = x[r] * n.cdf;
+        d[r] = n.cdf + x[r] * (0.39894228040143268f * n.e);
       }
       break;
     case ACT_RELU:
@@ -170,7 +199,7 @@ __device__ __forceinline__ void act_fwd_grad_w(int act, const float* x, float* y
     case ACT_TANH:
 #pragma unroll
       for (int r = 0; r < W; ++r) {
-        float t = tanhf(x[r]);
+        float t = tanh_f32(x[r]);
         y[r] = t;
         d[r] = 1.0f - t * t;
       }
