@@ -148,14 +148,16 @@ def _other_configs(dev):
 
 def _edge_shapes(dev):
     """Shapes off the tile grid, next to torch's own operators (rocBLAS/hipBLASLt) on the same GPU:
-    a ragged token count at the headline widths (fwd+bwd) and a short batch at the decode widths
-    (forward; the down projection splits its reduction)."""
+    a ragged token count at the headline widths (fwd+bwd), a short batch at the decode widths
+    (forward; the down projection splits its reduction) and a batch whose 2.3 GB activations are
+    beyond 32-bit byte offsets (fwd+bwd; the module runs it as two row chunks)."""
     from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP
 
     out = {}
     for name, (m, k, n, bwd) in {
         "ragged_fp16_fwdbwd_M8191_K4096_N14336": (8191, 4096, 14336, True),
         "short_batch_fp16_fwd_M32_K8192_N28672": (32, 8192, 28672, False),
+        "tall_batch_fp16_fwdbwd_M40960_K8192_N28672": (40960, 8192, 28672, True),
     }.items():
         fused = FusedGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
         eager = EagerGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
@@ -175,7 +177,8 @@ def _edge_shapes(dev):
                     with torch.no_grad():
                         mod(x)
 
-            res[label] = round(_event_time_ms(step, 10, warmup=3)[1], 4)
+            reps = 10 if m <= 8192 else 3
+            res[label] = round(_event_time_ms(step, reps, warmup=min(3, reps))[1], 4)
         flop = (18.0 if bwd else 6.0) * m * n * k
         res["tflops"] = round(flop / res["ms"] / 1e9, 1)
         out[name] = res

@@ -549,6 +549,18 @@ def test_many_tokens_tall_shape():
     _run_module_case(Case("tall_65536x256x512", 65536, 256, 512, torch.float16, bias=False, backward=True, seed=8))
 
 
+def test_batches_beyond_32bit_offsets_run_as_row_chunks(monkeypatch):
+    """A batch whose [M, N] activations exceed the pipelined kernels' 32-bit byte offsets is split
+    into row chunks by the module (here the limit is lowered to 512 rows: three chunks, the last one
+    ragged); outputs and all gradients, weight gradients summed over the chunks, match the oracle."""
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    assert ops_fwd.max_rows_32bit(8192, 28672, torch.float16) * 28672 * 2 < 2**31
+    monkeypatch.setattr(ops_fwd, "max_rows_32bit", lambda K, N, dtype: 512)
+    _run_module_case(Case("chunked_1300x256x640", 1300, 256, 640, torch.float16, bias=True, backward=True, seed=31))
+    _run_module_case(Case("chunked_1024x256x640", 1024, 256, 640, torch.bfloat16, bias=False, backward=True, seed=32))
+
+
 def test_memory_lean_backward_is_bit_identical():
     """recompute_activations=True (keep x only, as the reference does) gives the same gradients."""
     from triton_gated_mlp import FusedGatedMLP

@@ -230,3 +230,21 @@ def test_small_helpers_of_the_reference_surface():
     assert utils.validate_contiguous(a.T).is_contiguous() and torch.equal(utils.validate_contiguous(a.T), a.T)
     with pytest.raises(RuntimeError, match="GPU"):
         utils.validate_tensor_device(a)
+
+
+def test_max_rows_32bit_keeps_padded_operands_below_2_gib():
+    """The module's chunk size for very tall batches: a multiple of 256 whose [rows, max(K, N)]
+    operand, padded to whole 256-tiles, stays addressable with 32-bit byte offsets, and the next
+    multiple of 256 does not."""
+    from triton_gated_mlp.ops.fwd import max_rows_32bit
+
+    limit = (1 << 31) - 4096
+    for K, N in [(4096, 14336), (8192, 28672), (4096, 11008), (5120, 13824), (8, 8), (100, 72)]:
+        for dtype in (torch.float16, torch.bfloat16):
+            rows = max_rows_32bit(K, N, dtype)
+            width = -(-max(K, N) // 256) * 256
+            assert rows % 256 == 0 and rows >= 256
+            assert rows * width * 2 < limit
+            assert (rows + 256) * width * 2 >= limit
+    assert max_rows_32bit(8192, 28672, torch.float16) == 37376
+    assert max_rows_32bit(4096, 14336, torch.float32) is None

@@ -252,6 +252,19 @@ class FusedGatedMLP(_GatedMLPBase):
 
     def _forward_2d(self, x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p: float) -> Tensor:
         M, K = x2.shape
+        limit = _fwd.max_rows_32bit(K, self.intermediate_size, x2.dtype) if x2.is_cuda else None
+        if limit is not None and M > limit:
+            # Token rows are independent: a batch too tall for the pipelined kernels' 32-bit operand
+            # offsets runs as near-equal row chunks (autograd sums the chunks' weight gradients; with
+            # dropout every chunk draws its own mask and `last_dropout_state` is the last chunk's).
+            chunks = -(-M // limit)
+            rows = -(-M // (chunks * 256)) * 256
+            return torch.cat(
+                [
+                    self._forward_2d(x2[i : i + rows], W_gate, b_gate, W_up, b_up, W_down, b_down, p)
+                    for i in range(0, M, rows)
+                ]
+            )
         inference = not torch.is_grad_enabled() or not (
             x2.requires_grad or any(q.requires_grad for q in self.parameters())
         )

@@ -130,6 +130,21 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
 DECODE_MAX_M = 16
 
 
+def max_rows_32bit(K: int, N: int, dtype: torch.dtype) -> Optional[int]:
+    """Largest token count (a multiple of 256) whose [M, K] and [M, N] operands the pipelined kernels
+    can address, or None when there is no such limit (float32).
+
+    Those kernels read their operands through buffer descriptors with 32-bit byte offsets, padded
+    to whole tiles; the library runs anything larger on its slower predicated kernels.  Rows of the
+    MLP are independent, so the module splits such a batch into row chunks instead.
+    """
+    if dtype == torch.float32:
+        return None
+    width = (max(K, N) + 255) // 256 * 256
+    limit = (1 << 31) - 4096  # the descriptor base sits up to 4 KB below the operand
+    return max(256, (limit - 1) // (2 * width) // 256 * 256)
+
+
 def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16) -> bool:
     return dtype in (torch.float16, torch.bfloat16) and 1 <= M <= DECODE_MAX_M and K % 32 == 0 and N % 256 == 0
 
