@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 4
+#define GMLP_ABI_VERSION 5
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -177,7 +177,8 @@ int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void*
 
 /*
  * Skinny-M forward of the whole MLP (decode): y = (act(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
- * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch is [M,N] in dtype;
+ * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch holds 16*N elements
+ * of dtype: the intermediate H for 16 token slots, in an order of the library's choosing;
  * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
  * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
  * Requires K % 32 == 0 and N % 256 == 0 (the LDS-ring streaming kernels run when K % 256 == 0 too).

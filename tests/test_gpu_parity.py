@@ -605,7 +605,7 @@ def test_decode_matches_general_path():
     dev = _dev()
     g = torch.Generator().manual_seed(2)
     for M, K, N, bias in [(16, 1024, 2048, True), (3, 256, 512, False), (1, 4096, 11008, True), (5, 768, 1792, True),
-                          (16, 4096, 11008, False)]:
+                          (16, 4096, 11008, False), (12, 1024, 2048, True), (11, 768, 1792, False)]:
         x = torch.randn(M, K, generator=g).half().to(dev)
         Wg = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
         Wu = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)

@@ -50,6 +50,9 @@ constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
 // ring slots per wavefront (and stages in flight): 3 slots of two 16-row regions, or 4 of one
 constexpr int ds_ring_depth(int nmat) { return nmat == 2 ? 3 : 4; }
 constexpr int DS_WAVES = 3;           // wavefronts per workgroup
+#ifndef GMLP_DECODE_TILED_MIN
+#define GMLP_DECODE_TILED_MIN 10
+#endif
 
 struct StreamArgs {
   const void* x;      // [M, ldx] token rows (x or H)
@@ -58,6 +61,7 @@ struct StreamArgs {
   void* out;          // [M, ldo]
   int M, R, red, ldx, ldo;
   int act;            // Act code (GATED only)
+  int tiled;          // H (GATED: out, otherwise: x) is in fragment order, see ds_h_tiled()
 };
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -107,6 +111,11 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   const int spb = (chunks * (wave + 1)) / DS_WAVES - c0;
   const int my_blocks = (nblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
   const int total = my_blocks * spb;
+  // Workgroup b starts each block at chunk b % spb of its wavefronts' ranges and wraps around (a
+  // sum does not mind the order).  Without it every workgroup on the chip reads the same offset
+  // along its rows at the same time, and for a power-of-two row pitch (W_gate, W_up of the usual
+  // hidden sizes) those addresses crowd onto a few memory channels: 154 -> 142 us at K = 8192.
+  const int rot = (int)blockIdx.x % spb;
 
   // Per-lane byte offsets: weights, 8 load instructions per region (2 rows x 512 bytes each);
   // token operands, the 16 bytes of row lane%16 this lane feeds to each of the stage's 8 MFMAs.
@@ -117,10 +126,14 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     int row = 2 * q + (lane >> 5), pos = lane & 31;
     woff[q] = (uint32_t)(row * a.red + (pos ^ row) * 8) * 2u;
   }
-  {
-    int xr = r16 < a.M ? r16 : a.M - 1;  // rows past M repeat the last token row (never stored)
+  const bool tiled_x = !GATED && a.tiled;
+  if (tiled_x) {
+    xoff = (uint32_t)lane * 16u;  // a fragment is one contiguous KiB
+  } else {
+    int xr = r16 < a.M ? r16 : a.M - 1;  // rows past M repeat the last token row
     xoff = (uint32_t)(xr * a.ldx + kg * 8) * 2u;
   }
+  const uint32_t xq = tiled_x ? 1024u : 64u;  // from one MFMA's token operand to the next
   const buffer_rsrc rx = make_rsrc(a.x);
   const buffer_rsrc rw[2] = {make_rsrc(a.w[0]), make_rsrc(a.w[1])};
 
@@ -130,10 +143,15 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   auto issue_stage = [&](int i_req, int u) __attribute__((always_inline)) {
     int i = i_req < total ? i_req : total - 1;
     int j = i / spb, c = i - j * spb;
+    c += rot;
+    c = c < spb ? c : c - spb;
     int rb = (int)blockIdx.x + j * (int)gridDim.x;
     uint32_t koff = (uint32_t)((c0 + c) * DS_CH) * 2u;
+    // token operand of the stage's q-th MFMA: 64 bytes further along each row of x, or the next
+    // 1 KiB fragment of H (a stage of 256 elements x 16 token slots is 8 KiB)
+    const uint32_t xstage = tiled_x ? koff * 16u : koff;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) xf[u][q] = load16_async(rx, xoff, koff + q * 64);
+    for (int q = 0; q < 8; ++q) xf[u][q] = load16_async(rx, xoff, xstage + q * xq);
     uint32_t slot = lds_base + (uint32_t)u * SLOT;
     uint32_t woffs = (uint32_t)rb * (uint32_t)BLOCK_ROWS * (uint32_t)a.red * 2u + koff;
 #pragma unroll
@@ -184,7 +202,7 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
           __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-          if (wave == 0 && r16 < a.M) {
+          if (wave == 0 && ((GATED && a.tiled) || r16 < a.M)) {
             int rb = (int)blockIdx.x + blk * (int)gridDim.x;
             int r0 = rb * BLOCK_ROWS + 4 * kg;
             float v[NMAT][4];
@@ -205,7 +223,14 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
               act_fwd_w<4>(a.act, v[0], res);
 #pragma unroll
               for (int r = 0; r < 4; ++r) res[r] *= v[NMAT - 1][r];
-              store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
+              // Fragment order: H goes out the way the down projection's MFMAs take it in,
+              // [N/8][16 token slots][8 elements], so that a token-operand fragment there is one
+              // contiguous KiB instead of 16 row pieces of 64 bytes.  All 16 slots are written
+              // (slots past M repeat the last token), so nothing uninitialised is multiplied.
+              if (a.tiled)
+                store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * 16 + r16) * 8 + (r0 & 7), res);
+              else
+                store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
             } else {
 #pragma unroll
               for (int m = 0; m < NMAT; ++m) store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16 * m, v[m]);
@@ -233,6 +258,11 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
   return hipGetLastError();
 }
 
+// Layout of the intermediate H between the two kernels.  Row-major [M, N] costs the down projection
+// M pieces of 64 bytes per token-operand fragment, fragment order always one KiB (16 token slots):
+// cheaper from about half-full upwards.
+static int ds_h_tiled(int M) { return M > GMLP_DECODE_TILED_MIN ? 1 : 0; }
+
 bool decode_stream_supported(int M, int K, int N) {
   return M >= 1 && M <= 16 && K % DS_CH == 0 && N % DS_CH == 0 && K >= DS_WAVES * DS_CH && N >= DS_WAVES * DS_CH &&
          (int64_t)K * N * 2 < ((int64_t)1 << 31);
@@ -246,10 +276,11 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
   if (hipError_t e = hipGetDevice(&dev)) return e;
   if (hipError_t e = hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev)) return e;
   if (num_cu <= 0) num_cu = 256;
-  StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act};
+  const int tiled = ds_h_tiled(M);
+  StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act, tiled};
   hipError_t e = launch_stream<T, true, 2>(a1, num_cu, s);
   if (e != hipSuccess) return e;
-  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY};
+  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY, tiled};
   // 32-row blocks halve the L2 traffic for H, but only pay when they still occupy every CU
   if (K / 32 >= num_cu) return launch_stream<T, false, 2>(a2, num_cu, s);
   return launch_stream<T, false, 1>(a2, num_cu, s);

@@ -152,15 +152,24 @@ def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16)
 def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16, num_cu: int = 256) -> bool:
     """True when the skinny-M streaming kernels are the faster way to run the forward pass.
 
-    They hand out 16 rows of W_gate/W_up and 16 or 32 rows of W_down per workgroup and step.  With
-    at least one 32-row block per compute unit (both widths >= 32 * num_cu) they win for every
-    M <= 16; down to half that hidden size they still win for M <= 8; below, the general path
-    (GEMMs with split reductions) is as fast or faster.  Measured on MI355X at the widths of
-    Llama-2-7B/13B, Llama-3-8B and Llama-3-70B.
+    They hand out blocks of 16 rows of W_gate/W_up, and of 32 (or 16) rows of W_down, to one
+    workgroup per compute unit.  They need at least one block of W_gate/W_up rows per unit; from
+    there they beat the general path (GEMMs with split reductions) for every M <= 8, and for
+    M <= 16 as long as the blocks divide over the units without leaving too many of them idle in
+    the last round (measured on MI355X at the widths of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384
+    and 2048 x 8192; Llama-2-13B's 864 and 320 blocks over 256 units are the case that loses).
     """
-    if not (decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 32 * num_cu):
+    if not (decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu):
         return False
-    return K >= 32 * num_cu or (M <= 8 and K >= 16 * num_cu)
+    if M <= 8:
+        return True
+
+    def fill(blocks: int) -> float:
+        return blocks / (-(-blocks // num_cu) * num_cu)
+
+    gate_up = fill(N // 16)  # streams two thirds of the bytes
+    down = fill(K // 32 if K // 32 >= num_cu else K // 16)
+    return 3.0 / (2.0 / gate_up + 1.0 / down) >= 0.85
 
 
 def decode_fwd(
@@ -184,7 +193,7 @@ def decode_fwd(
     act = _cabi.act_code(act_fn)
     x, W_gate, W_up, W_down = _c(x), _c(W_gate), _c(W_up), _c(W_down)
     b_gate, b_up, b_down = _c(b_gate), _c(b_up), _c(b_down)
-    h = torch.empty((M, N), dtype=x.dtype, device=dev)
+    h = torch.empty((16, N), dtype=x.dtype, device=dev)  # scratch: H for 16 token slots, library's layout
     y = torch.empty((M, K), dtype=x.dtype, device=dev)
     with torch.cuda.device(dev):
         _cabi.check(
