@@ -6,9 +6,10 @@ N=14336 (Llama-3-8B MLP), bias=False, dropout_p=0; one step = `y = mlp(x); y.bac
 dense upstream gradient.  FLOP model: 18*M*N*K per step (3 forward + 6 backward GEMMs), the same
 count as the reference's `9 * 2 * M * N * K` (src/triton_gated_mlp/benchmark.py:86).
 
-Prints ONE JSON line.  `roofline` covers the dominant kernel (the gate/up forward GEMM with the fused
-SiLU-gating epilogue, 4*M*N*K FLOP per launch) timed with events on the launch stream; `kernels`
-lists every launch of a step the same way; `cpu_baseline` times the CPU oracle on a bounded sample.
+Prints ONE JSON line.  `roofline` covers the dominant kernel (the grouped launch of the three
+weight-gradient GEMMs, a third of the step: 6*M*N*K FLOP per launch) timed with events on the launch
+stream; `kernels` lists every launch of a step the same way; `cpu_baseline` times the CPU oracle on
+a bounded sample.
 """
 
 from __future__ import annotations
@@ -32,7 +33,8 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 M, K, N = 8192, 4096, 14336
 DTYPE = torch.float16
 # rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain copy of known size reads) + WRITE_SIZE, per launch
-GATEUP_TRAFFIC_BYTES = 3.525e9
+# of the grouped weight-gradient kernel: 2 183 357 KiB x 2.0 + 344 064 KiB
+DW_GROUP_TRAFFIC_BYTES = 4.824e9
 
 
 def _median(v):
@@ -265,19 +267,24 @@ def main():
     flop_step = 18.0 * M * N * K
     tflops = flop_step / (ms_per_step * 1e-3) / 1e12
 
-    # dominant kernel: gate/up forward GEMM (4*M*N*K FLOP per launch), events on the launch stream
+    # dominant kernel: dW_gate, dW_up and dW_down as one grouped launch (6*M*N*K FLOP), events on
+    # the launch stream
+    from triton_gated_mlp.ops import bwd as B
     from triton_gated_mlp.ops import fwd as F
 
-    Wg, Wu = mlp.gate_proj.weight.detach(), mlp.up_proj.weight.detach()
+    Wg, Wu, Wd = mlp.gate_proj.weight.detach(), mlp.up_proj.weight.detach(), mlp.down_proj.weight.detach()
     xd = x.detach()
-    avg, med = _event_time_ms(lambda: F.gateup_fwd(xd, Wg, None, Wu, None, save_activations=True), max(args.steps, 10))
-    dom_flop = 4.0 * M * N * K
-    roofline = {"kernel": "gemm_kernel_pipelined<f16,256,128,16,...,EpiGateUp> (gate/up forward GEMM + SiLU-gating epilogue)",
+    hs = F.gateup_fwd(xd, Wg, None, Wu, None, save_activations=True)
+    dg, du = B.dh_bwd(dY, Wd, hs.gate, hs.up)
+    avg, med = _event_time_ms(lambda: B.dw_bwd_grouped([(dg, xd), (du, xd), (dY, hs.hidden)]), max(args.steps, 10))
+    del dg, du, hs
+    dom_flop = 6.0 * M * N * K
+    roofline = {"kernel": "gemm_group_kernel_pipelined<f16,256,256,16,...,EpiStore> (dW_gate + dW_up + dW_down, one grouped launch)",
                 "bound": "mfma", "achieved": round(dom_flop / avg / 1e9, 1), "peak": PEAK_MFMA_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_flop / avg / 1e9 / PEAK_MFMA_F16_TFLOPS, 4),
-                "avg_launch_ms": round(avg, 4), "flop_per_launch": dom_flop, "traffic": GATEUP_TRAFFIC_BYTES,
+                "avg_launch_ms": round(avg, 4), "flop_per_launch": dom_flop, "traffic": DW_GROUP_TRAFFIC_BYTES,
                 "traffic_note": "HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
-                                "(profiles/gateup_gemm_hbm_traffic.txt); algorithmic bytes are 1.007e9"}
+                                "(profiles/gemm_hbm_traffic_fp16_M8192_K4096_N14336.txt); algorithmic bytes are 1.258e9"}
 
     line = {
         "metric": "fwd+bwd TFLOP/s & % MFMA peak, fp16 M=8192 K=4096 N=14336 (1 GPU)",
