@@ -599,22 +599,26 @@ def test_grouped_weight_gradients_equal_single_launches():
         _close("dW_gate grouped", grouped[0], dg.float().cpu().T @ x.float().cpu(), atol=ATOL * 40)
 
 
-def test_decode_matches_general_path():
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decode_matches_general_path(dtype):
+    """Skinny-M kernels against the oracle and the general path: both layouts of the intermediate H
+    (row-major up to M = 10, fragment order above, with token slots past M), both streaming variants
+    of the down projection, and shapes that only the register-streaming kernels take."""
     from triton_gated_mlp.ops import fwd as ops_fwd
 
     dev = _dev()
     g = torch.Generator().manual_seed(2)
     for M, K, N, bias in [(16, 1024, 2048, True), (3, 256, 512, False), (1, 4096, 11008, True), (5, 768, 1792, True),
-                          (16, 4096, 11008, False), (12, 1024, 2048, True), (11, 768, 1792, False)]:
-        x = torch.randn(M, K, generator=g).half().to(dev)
-        Wg = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
-        Wu = (0.02 * torch.randn(N, K, generator=g)).half().to(dev)
-        Wd = (0.02 * torch.randn(K, N, generator=g)).half().to(dev)
+                          (16, 4096, 11008, False), (12, 1024, 2048, True), (11, 768, 1792, False), (10, 8192, 512, True)]:
+        x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+        Wg = (0.02 * torch.randn(N, K, generator=g)).to(dtype).to(dev)
+        Wu = (0.02 * torch.randn(N, K, generator=g)).to(dtype).to(dev)
+        Wd = (0.02 * torch.randn(K, N, generator=g)).to(dtype).to(dev)
         bg = bu = bd = None
         if bias:
-            bg = (0.01 * torch.randn(N, generator=g)).half().to(dev)
-            bu = (0.01 * torch.randn(N, generator=g)).half().to(dev)
-            bd = (0.01 * torch.randn(K, generator=g)).half().to(dev)
+            bg = (0.01 * torch.randn(N, generator=g)).to(dtype).to(dev)
+            bu = (0.01 * torch.randn(N, generator=g)).to(dtype).to(dev)
+            bd = (0.01 * torch.randn(K, generator=g)).to(dtype).to(dev)
         y = ops_fwd.decode_fwd(x, Wg, bg, Wu, bu, Wd, bd)
         f = lambda t: None if t is None else t.float().cpu()
         ref = oracle.forward(f(x), f(Wg), f(bg), f(Wu), f(bu), f(Wd), f(bd))
