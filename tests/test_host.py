@@ -250,15 +250,14 @@ def test_max_rows_32bit_keeps_padded_operands_below_2_gib():
     assert max_rows_32bit(4096, 14336, torch.float32) is None
 
 
-def test_decode_preferred_follows_the_block_balance():
+def test_decode_preferred_needs_widths_that_fill_the_chip():
     """Routing of M <= 16 inference between the streaming kernels and the general path."""
     from triton_gated_mlp.ops.fwd import decode_preferred
 
-    for K, N in [(8192, 28672), (4096, 14336), (4096, 11008), (6144, 16384)]:
+    for K, N in [(8192, 28672), (4096, 14336), (4096, 11008), (5120, 13824), (6144, 16384), (2048, 8192)]:
         assert all(decode_preferred(M, K, N) for M in (1, 8, 9, 16)), (K, N)
-    assert decode_preferred(8, 5120, 13824) and not decode_preferred(12, 5120, 13824)  # 864 and 320 blocks on 256 units
-    assert decode_preferred(4, 2048, 8192) and not decode_preferred(16, 2048, 8192)
     assert not decode_preferred(17, 8192, 28672)  # beyond the skinny-M kernels
     assert not decode_preferred(1, 4096 + 64, 14336)  # K must be a multiple of 256 for the streaming kernels
     assert not decode_preferred(1, 1024, 2048)  # fewer W_gate/W_up blocks than compute units
+    assert not decode_preferred(1, 1024, 8192)  # a quarter of a W_down block per compute unit
     assert not decode_preferred(1, 8192, 28672, torch.float32)

@@ -1,10 +1,11 @@
 // Skinny-M (M <= 16) weight-streaming kernels, HBM-bound: every weight byte is fetched once, in
 // 512-byte row segments moved global -> LDS without passing through registers.
 //
-// One persistent workgroup of three wavefronts per CU.  The workgroup owns blocks of 2 x 16 weight
-// rows (rb = blockIdx.x, blockIdx.x + gridDim.x, ...) that share one set of token operands: rows
-// r..r+15 of W_gate and of W_up (GATED), or 32 consecutive rows of W_down (16 when the hidden size
-// gives fewer than one 32-row block per CU); its wavefronts split the reduction range in
+// One persistent workgroup of three wavefronts per CU.  The workgroup takes blocks of weight rows
+// that share one set of token operands: rows r..r+15 of W_gate and of W_up (GATED), or 32
+// consecutive rows of W_down (16 when a CU's share is no more than that); whole blocks go round-robin
+// over the workgroups, the rows that do not fill a last round are shared out evenly as one partly
+// empty block each.  Its wavefronts split the reduction range in
 // near-equal runs of 256-element chunks and combine their partial sums through LDS at the
 // end of each block (fixed order, so the result is deterministic).  Each wavefront runs a private
 // ring of 3 LDS slots; a slot holds one stage = 256 reduction elements of the 16 weight rows of
@@ -50,6 +51,7 @@ constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
 // ring slots per wavefront (and stages in flight): 3 slots of two 16-row regions, or 4 of one
 constexpr int ds_ring_depth(int nmat) { return nmat == 2 ? 3 : 4; }
 constexpr int DS_WAVES = 3;           // wavefronts per workgroup
+constexpr uint32_t DS_NOWHERE = 0x80000000u;  // voffset beyond any operand (operands are < 2 GiB)
 #ifndef GMLP_DECODE_TILED_MIN
 #define GMLP_DECODE_TILED_MIN 10
 #endif
@@ -104,12 +106,33 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   char* ring = smem + wave * (DS_RD * SLOT);
   float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [2 parities][waves-1][NMAT][64][4]
 
-  const int nblocks = a.R / BLOCK_ROWS;
+  // Blocks of BLOCK_ROWS weight rows go round-robin over the workgroups (block b, b + G, ...: at any
+  // time the chip streams one contiguous band of rows) for as many rounds as every workgroup gets a
+  // whole block.  The rows left over (the tail) are shared out evenly instead, in multiples of 4
+  // (what one lane stores), so that every CU streams the same number of bytes whatever R is: a
+  // workgroup's tail share [t_begin, t_end) is one last block with fewer valid rows, the loads of
+  // the others go nowhere (an offset beyond the descriptor reads as zero and moves no data) and
+  // their results are not stored.
+  const int G = (int)gridDim.x;
+  const int full = a.R / BLOCK_ROWS / G;
+  const int tail0 = full * G * BLOCK_ROWS, tail_rows = a.R - tail0;
+  const int t_begin = tail0 + (((int)blockIdx.x * tail_rows / G) & ~3);
+  const int t_end = (int)blockIdx.x + 1 == G ? a.R : tail0 + ((((int)blockIdx.x + 1) * tail_rows / G) & ~3);
+  // first row and number of existing rows (BLOCK_ROWS or more: all) of this workgroup's j-th block
+  auto block_rows = [&](int j, int& row0, int& valid) __attribute__((always_inline)) {
+    if (j < full) {
+      row0 = ((int)blockIdx.x + j * G) * BLOCK_ROWS;
+      valid = BLOCK_ROWS;
+    } else {
+      row0 = t_begin + (j - full) * BLOCK_ROWS;
+      valid = t_end - row0;
+    }
+  };
   const int chunks = a.red / DS_CH;
   // wavefront w reduces chunks [c0, c0 + spb)
   const int c0 = (chunks * wave) / DS_WAVES;
   const int spb = (chunks * (wave + 1)) / DS_WAVES - c0;
-  const int my_blocks = (nblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int my_blocks = full + (t_end - t_begin + BLOCK_ROWS - 1) / BLOCK_ROWS;
   const int total = my_blocks * spb;
   // Workgroup b starts each block at chunk b % spb of its wavefronts' ranges and wraps around (a
   // sum does not mind the order).  Without it every workgroup on the chip reads the same offset
@@ -121,9 +144,11 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   // token operands, the 16 bytes of row lane%16 this lane feeds to each of the stage's 8 MFMAs.
   const int r16 = lane & 15, kg = lane >> 4;
   uint32_t woff[8], xoff;
+  int wrow[8];  // row of the region that load q of this lane fetches
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
     int row = 2 * q + (lane >> 5), pos = lane & 31;
+    wrow[q] = row;
     woff[q] = (uint32_t)(row * a.red + (pos ^ row) * 8) * 2u;
   }
   const bool tiled_x = !GATED && a.tiled;
@@ -135,7 +160,10 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   }
   const uint32_t xq = tiled_x ? 1024u : 64u;  // from one MFMA's token operand to the next
   const buffer_rsrc rx = make_rsrc(a.x);
-  const buffer_rsrc rw[2] = {make_rsrc(a.w[0]), make_rsrc(a.w[1])};
+  // exact sizes: w[1] is W_up (GATED) or W_down from its row 16 on
+  const uint32_t w_bytes = (uint32_t)a.R * (uint32_t)a.red * 2u;
+  const buffer_rsrc rw[2] = {make_rsrc(a.w[0], w_bytes),
+                             make_rsrc(a.w[1], GATED ? w_bytes : w_bytes - 16u * (uint32_t)a.red * 2u)};
 
   i32x4 xf[DS_RD][8];
 
@@ -145,7 +173,8 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     int j = i / spb, c = i - j * spb;
     c += rot;
     c = c < spb ? c : c - spb;
-    int rb = (int)blockIdx.x + j * (int)gridDim.x;
+    int row0, valid;
+    block_rows(j, row0, valid);
     uint32_t koff = (uint32_t)((c0 + c) * DS_CH) * 2u;
     // token operand of the stage's q-th MFMA: 64 bytes further along each row of x, or the next
     // 1 KiB fragment of H (a stage of 256 elements x 16 token slots is 8 KiB)
@@ -153,12 +182,14 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
 #pragma unroll
     for (int q = 0; q < 8; ++q) xf[u][q] = load16_async(rx, xoff, xstage + q * xq);
     uint32_t slot = lds_base + (uint32_t)u * SLOT;
-    uint32_t woffs = (uint32_t)rb * (uint32_t)BLOCK_ROWS * (uint32_t)a.red * 2u + koff;
+    uint32_t woffs = (uint32_t)row0 * (uint32_t)a.red * 2u + koff;
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m)
+    for (int m = 0; m < NMAT; ++m) {
+      const int valid_m = GATED ? valid : valid - 16 * m;
 #pragma unroll
       for (int q = 0; q < 8; ++q)
-        load16_to_lds<true>(rw[m], woff[q], woffs, slot + m * DS_REGION + q * 1024);
+        load16_to_lds<true>(rw[m], wrow[q] < valid_m ? woff[q] : DS_NOWHERE, woffs, slot + m * DS_REGION + q * 1024);
+    }
   };
 
   f32x4v acc[NMAT];
@@ -203,8 +234,9 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
           __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
           if (wave == 0 && ((GATED && a.tiled) || r16 < a.M)) {
-            int rb = (int)blockIdx.x + blk * (int)gridDim.x;
-            int r0 = rb * BLOCK_ROWS + 4 * kg;
+            int row0, valid;
+            block_rows(blk, row0, valid);
+            const int r0 = row0 + 4 * kg;  // this lane's four rows (of each region)
             float v[NMAT][4];
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
@@ -216,7 +248,8 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
 #pragma unroll
                 for (int r = 0; r < 4; ++r) v[m][r] += o[r];
               }
-              if (a.bias[m]) add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
+              if (a.bias[m] && 4 * kg + (GATED ? 0 : 16 * m) < valid)
+                add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
             }
             if (GATED) {
               float res[4];
@@ -227,13 +260,16 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
               // [N/8][16 token slots][8 elements], so that a token-operand fragment there is one
               // contiguous KiB instead of 16 row pieces of 64 bytes.  All 16 slots are written
               // (slots past M repeat the last token), so nothing uninitialised is multiplied.
-              if (a.tiled)
-                store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * 16 + r16) * 8 + (r0 & 7), res);
-              else
-                store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
+              if (4 * kg < valid) {
+                if (a.tiled)
+                  store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * 16 + r16) * 8 + (r0 & 7), res);
+                else
+                  store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
+              }
             } else {
 #pragma unroll
-              for (int m = 0; m < NMAT; ++m) store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16 * m, v[m]);
+              for (int m = 0; m < NMAT; ++m)
+                if (4 * kg + 16 * m < valid) store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16 * m, v[m]);
             }
           }
 #pragma unroll
@@ -252,8 +288,8 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
   auto kern = decode_stream_kernel<T, GATED, NMAT>;
   static LdsAttrOnce lds_attr;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
-  int nblocks = a.R / (GATED ? 16 : 16 * NMAT);
-  int grid = nblocks < num_cu ? nblocks : num_cu;
+  // one workgroup per CU, each with its share of the rows; fewer when that would be under 16 rows
+  int grid = a.R / 16 < num_cu ? a.R / 16 : num_cu;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);
   return hipGetLastError();
 }
@@ -281,8 +317,8 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
   hipError_t e = launch_stream<T, true, 2>(a1, num_cu, s);
   if (e != hipSuccess) return e;
   StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY, tiled};
-  // 32-row blocks halve the L2 traffic for H, but only pay when they still occupy every CU
-  if (K / 32 >= num_cu) return launch_stream<T, false, 2>(a2, num_cu, s);
+  // 32-row blocks halve the L2 traffic for H; worth it when a CU's share of the rows exceeds 16
+  if (K > 16 * num_cu) return launch_stream<T, false, 2>(a2, num_cu, s);
   return launch_stream<T, false, 1>(a2, num_cu, s);
 }
 

@@ -152,24 +152,13 @@ def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16)
 def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16, num_cu: int = 256) -> bool:
     """True when the skinny-M streaming kernels are the faster way to run the forward pass.
 
-    They hand out blocks of 16 rows of W_gate/W_up, and of 32 (or 16) rows of W_down, to one
-    workgroup per compute unit.  They need at least one block of W_gate/W_up rows per unit; from
-    there they beat the general path (GEMMs with split reductions) for every M <= 8, and for
-    M <= 16 as long as the blocks divide over the units without leaving too many of them idle in
-    the last round (measured on MI355X at the widths of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384
-    and 2048 x 8192; Llama-2-13B's 864 and 320 blocks over 256 units are the case that loses).
+    They give every compute unit the same share of the weight rows (in blocks of 16 rows of
+    W_gate/W_up, and of 32 or 16 rows of W_down), so they need widths that give each unit at least
+    a block of W_gate/W_up rows and half a block of W_down rows; from there they beat or match the
+    general path (GEMMs with split reductions) for every M <= 16 (measured on MI355X at the widths
+    of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384 and 2048 x 8192).
     """
-    if not (decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu):
-        return False
-    if M <= 8:
-        return True
-
-    def fill(blocks: int) -> float:
-        return blocks / (-(-blocks // num_cu) * num_cu)
-
-    gate_up = fill(N // 16)  # streams two thirds of the bytes
-    down = fill(K // 32 if K // 32 >= num_cu else K // 16)
-    return 3.0 / (2.0 / gate_up + 1.0 / down) >= 0.85
+    return decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu and K >= 8 * num_cu
 
 
 def decode_fwd(
