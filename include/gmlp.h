@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 5
+#define GMLP_ABI_VERSION 6
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -177,11 +177,13 @@ int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void*
 
 /*
  * Skinny-M forward of the whole MLP (decode): y = (act(x·W_gateᵀ+b_g) ⊙ (x·W_upᵀ+b_u))·W_downᵀ + b_d
- * for M <= 16, streaming each weight matrix from HBM exactly once.  h_scratch holds 16*N elements
- * of dtype: the intermediate H for 16 token slots, in an order of the library's choosing;
+ * for M <= 32, streaming each weight matrix from HBM exactly once.  h_scratch holds 16*N elements
+ * of dtype for M <= 16 and 32*N beyond: the intermediate H for 16 or 32 token slots, in an order of
+ * the library's choosing;
  * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
  * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
- * Requires K % 32 == 0 and N % 256 == 0 (the LDS-ring streaming kernels run when K % 256 == 0 too).
+ * Requires K % 32 == 0 and N % 256 == 0 (the LDS-ring streaming kernels run when K % 256 == 0 too,
+ * K >= 768, N >= 768 and K*N < 2^30; 16 < M <= 32 is accepted only then).
  */
 int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                     const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,

@@ -628,6 +628,39 @@ def test_decode_matches_general_path(dtype):
         _close(f"general Y M={M}", y_general, ref["Y"])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decode_with_two_token_tiles(dtype):
+    """16 < M <= 32 on the streaming kernels (two MFMAs per weight fragment, H for 32 token slots):
+    full and partly filled second tiles, both block heights of the down projection, widths whose
+    rows do not fill a last round of blocks, with and without biases."""
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(5)
+    for M, K, N, bias in [(32, 1024, 2048, True), (17, 768, 1792, False), (24, 8192, 768, True), (31, 4096, 11008, True),
+                          (20, 4352, 1024, False), (32, 5120, 13824, False)]:
+        assert ops_fwd.decode_supported(M, K, N, dtype)
+        print(f"decode two tiles {dtype} M={M} K={K} N={N} bias={bias}", flush=True)
+        x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+        Wg = (0.02 * torch.randn(N, K, generator=g)).to(dtype).to(dev)
+        Wu = (0.02 * torch.randn(N, K, generator=g)).to(dtype).to(dev)
+        Wd = (0.02 * torch.randn(K, N, generator=g)).to(dtype).to(dev)
+        bg = bu = bd = None
+        if bias:
+            bg = (0.01 * torch.randn(N, generator=g)).to(dtype).to(dev)
+            bu = (0.01 * torch.randn(N, generator=g)).to(dtype).to(dev)
+            bd = (0.01 * torch.randn(K, generator=g)).to(dtype).to(dev)
+        y = ops_fwd.decode_fwd(x, Wg, bg, Wu, bu, Wd, bd)
+        f = lambda t: None if t is None else t.float().cpu()
+        ref = oracle.forward(f(x), f(Wg), f(bg), f(Wu), f(bu), f(Wd), f(bd))
+        _close(f"decode Y M={M}", y, ref["Y"])
+    # shapes the streaming kernels do not take keep the limit of 16 rows
+    assert not ops_fwd.decode_supported(17, 512, 1024, dtype)
+    with pytest.raises(NotImplementedError):
+        ops_fwd.decode_fwd(torch.zeros(17, 512, dtype=dtype, device=dev), *[t for _ in range(2) for t in (torch.zeros(1024, 512, dtype=dtype, device=dev), None)],
+                           torch.zeros(512, 1024, dtype=dtype, device=dev), None)
+
+
 @pytest.mark.parametrize("M,K,N", [(8, 1024, 4096), (64, 1024, 4096)])
 def test_inference_forward_under_hip_graph_replay(M, K, N):
     """Serving loops replay a captured forward: the skinny-M streaming path (M = 8) and the general

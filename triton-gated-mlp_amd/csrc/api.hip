@@ -484,7 +484,11 @@ int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const v
   GMLP_REQUIRE_ACT(act);
   if (int rc = check_dims(__func__, M, K, N)) return rc;
   if (dtype == GMLP_F32) return fail(GMLP_ESHAPE, "%s: float32 is not supported by the skinny-M kernels", __func__);
-  if (M > 16) return fail(GMLP_ESHAPE, "%s: M = %lld exceeds the skinny-M limit of 16", __func__, (long long)M);
+  if (M > 32 || (M > 16 && !decode_stream_supported((int)M, (int)K, (int)N)))
+    return fail(GMLP_ESHAPE,
+                "%s: M = %lld exceeds the skinny-M limit (32 when K and N are multiples of 256, at least 768, "
+                "and K*N < 2^30; 16 otherwise)",
+                __func__, (long long)M);
   if (K % 32 != 0) return fail(GMLP_ESHAPE, "%s: K = %lld must be a multiple of 32", __func__, (long long)K);
   if (N % 256 != 0) return fail(GMLP_ESHAPE, "%s: N = %lld must be a multiple of 256", __func__, (long long)N);
   GMLP_REQUIRE_ALIGNED(x); GMLP_REQUIRE_ALIGNED(w_gate); GMLP_REQUIRE_ALIGNED(w_up);

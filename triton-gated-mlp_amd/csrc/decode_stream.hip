@@ -1,4 +1,4 @@
-// Skinny-M (M <= 16) weight-streaming kernels, HBM-bound: every weight byte is fetched once, in
+// Skinny-M (M <= 32) weight-streaming kernels, HBM-bound: every weight byte is fetched once, in
 // 512-byte row segments moved global -> LDS without passing through registers.
 //
 // One persistent workgroup of three wavefronts per CU.  The workgroup takes blocks of weight rows
@@ -10,7 +10,8 @@
 // end of each block (fixed order, so the result is deterministic).  Each wavefront runs a private
 // ring of 3 LDS slots; a slot holds one stage = 256 reduction elements of the 16 weight rows of
 // each matrix.  The matching token-row operands (x or H, L2-resident) are fetched straight into
-// registers, three stages ahead as well.  Achieved HBM bandwidth follows the bytes in flight per
+// registers, three stages ahead as well: one 16-token tile for M <= 16, two beyond (MT; the weight
+// fragment read from LDS then feeds two MFMAs).  Achieved HBM bandwidth follows the bytes in flight per
 // CU, and LDS capacity bounds those: wavefronts x 3 slots x slot size fill 144 of the 160 KiB.
 // The stream of stages runs on across block boundaries, so the ring never drains; loads past the
 // end re-fetch the last stage into a free slot, which keeps the in-flight count constant.
@@ -49,7 +50,8 @@ struct Mfma16x<bf16> {
 constexpr int DS_CH = 256;            // reduction elements per stage
 constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
 // ring slots per wavefront (and stages in flight): 3 slots of two 16-row regions, or 4 of one
-constexpr int ds_ring_depth(int nmat) { return nmat == 2 ? 3 : 4; }
+// (3 with two token tiles: the token operands in flight are bounded by the registers, see below)
+constexpr int ds_ring_depth(int nmat, int mt) { return nmat == 2 || mt == 2 ? 3 : 4; }
 constexpr int DS_WAVES = 3;           // wavefronts per workgroup
 constexpr uint32_t DS_NOWHERE = 0x80000000u;  // voffset beyond any operand (operands are < 2 GiB)
 #ifndef GMLP_DECODE_TILED_MIN
@@ -77,34 +79,52 @@ __device__ __forceinline__ i32x4 load16_async(buffer_rsrc r, uint32_t voffset, u
                : "memory");
   return v;
 }
-// s_waitcnt vmcnt(N) that also "defines" the 8 registers a stage's token operands arrive in, so
-// no use of them can be scheduled above the wait.
-template <int N>
-__device__ __forceinline__ void wait_vmem_keep(i32x4 (&x)[8]) {
+// s_waitcnt vmcnt(N) that also "defines" the registers a stage's token operands arrive in (8 per
+// token tile), so no use of them can be scheduled above the wait.  The second statement issues no
+// instruction: volatile asm statements keep their order, so it ties the second tile's registers
+// to the same point.
+template <int N, int NX>
+__device__ __forceinline__ void wait_vmem_keep(i32x4 (&x)[NX]) {
+  static_assert(NX == 8 || NX == 16, "one or two token tiles");
   asm volatile("s_waitcnt vmcnt(%8)"
                : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]),
                  "+v"(x[7])
                : "n"(N)
                : "memory");
+  if constexpr (NX == 16)
+    asm volatile(""
+                 : "+v"(x[8]), "+v"(x[9]), "+v"(x[10]), "+v"(x[11]), "+v"(x[12]), "+v"(x[13]),
+                   "+v"(x[14]), "+v"(x[15])
+                 :
+                 : "memory");
 }
 
 // NMAT: 16-row regions per stage (GATED: W_gate and W_up; otherwise 1 or 2 runs of W_down rows).
-template <typename T, bool GATED, int NMAT>
+// MT: tiles of 16 token slots (M <= 16 * MT).
+template <typename T, bool GATED, int NMAT, int MT>
 __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs a) {
   typedef typename Traits<T>::vec8 vec8;
   static_assert(NMAT == 2 || (NMAT == 1 && !GATED), "gated blocks stream two matrices");
-  constexpr int DS_RD = ds_ring_depth(NMAT);
+  constexpr int DS_RD = ds_ring_depth(NMAT, MT);
+  // The token operands in flight live in VGPRs that the loads fill asynchronously.  Were there not
+  // enough of the 256 left beside them, the compiler would park them elsewhere right after the
+  // load instruction, before the data has arrived.
+  static_assert(DS_RD * 8 * MT * 4 <= 192, "token operands in flight must leave room in the VGPRs");
   constexpr int BLOCK_ROWS = GATED ? 16 : 16 * NMAT;  // weight rows (per matrix) a block advances by
   constexpr int SLOT = NMAT * DS_REGION;
-  constexpr int LPS = 8 + 8 * NMAT;  // load instructions per stage (token operands + weights)
-  static_assert((DS_RD - 1) * LPS < 64, "the younger stages must fit the 6-bit vmcnt");
+  constexpr int LPS = 8 * MT + 8 * NMAT;  // load instructions per stage (token operands + weights)
+  // A stage is complete when no more than the DS_RD - 1 younger stages are in flight.  vmcnt has 6
+  // bits: where that count exceeds 63 the wait also covers the first token-operand loads of the
+  // next stage (issued right behind the awaited weights, and loads return in order).
+  constexpr int YOUNGER = (DS_RD - 1) * LPS < 63 ? (DS_RD - 1) * LPS : 63;
+  static_assert((DS_RD - 1) * LPS - YOUNGER <= 8 * MT, "the wait may only reach into the next stage's token operands");
 
   extern __shared__ __align__(1024) char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem + wave * (DS_RD * SLOT);
   char* ring = smem + wave * (DS_RD * SLOT);
-  float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [2 parities][waves-1][NMAT][64][4]
+  float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [2 parities][waves-1][NMAT][MT][64][4]
 
   // Blocks of BLOCK_ROWS weight rows go round-robin over the workgroups (block b, b + G, ...: at any
   // time the chip streams one contiguous band of rows) for as many rounds as every workgroup gets a
@@ -141,9 +161,9 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   const int rot = (int)blockIdx.x % spb;
 
   // Per-lane byte offsets: weights, 8 load instructions per region (2 rows x 512 bytes each);
-  // token operands, the 16 bytes of row lane%16 this lane feeds to each of the stage's 8 MFMAs.
+  // token operands, the 16 bytes of token row 16 t + lane%16 this lane feeds to the MFMAs of tile t.
   const int r16 = lane & 15, kg = lane >> 4;
-  uint32_t woff[8], xoff;
+  uint32_t woff[8], xoff[MT];
   int wrow[8];  // row of the region that load q of this lane fetches
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
@@ -152,20 +172,27 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     woff[q] = (uint32_t)(row * a.red + (pos ^ row) * 8) * 2u;
   }
   const bool tiled_x = !GATED && a.tiled;
-  if (tiled_x) {
-    xoff = (uint32_t)lane * 16u;  // a fragment is one contiguous KiB
-  } else {
-    int xr = r16 < a.M ? r16 : a.M - 1;  // rows past M repeat the last token row
-    xoff = (uint32_t)(xr * a.ldx + kg * 8) * 2u;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (tiled_x) {
+      // [red/8][16 MT token slots][8 elements]: the 8-element group kg of a fragment is 256 MT
+      // bytes after the previous one (for MT = 1 a fragment is one contiguous KiB)
+      xoff[t] = (uint32_t)(kg * (256 * MT) + t * 256 + r16 * 16);
+    } else {
+      int xr = 16 * t + r16 < a.M ? 16 * t + r16 : a.M - 1;  // rows past M repeat the last token row
+      xoff[t] = (uint32_t)(xr * a.ldx + kg * 8) * 2u;
+    }
   }
-  const uint32_t xq = tiled_x ? 1024u : 64u;  // from one MFMA's token operand to the next
-  const buffer_rsrc rx = make_rsrc(a.x);
+  const uint32_t xq = tiled_x ? 1024u * MT : 64u;  // from one MFMA's token operand to the next
+  // exact size: an offset past the end reads as zero instead of touching memory
+  const buffer_rsrc rx = make_rsrc(a.x, tiled_x ? (uint32_t)(16 * MT) * (uint32_t)a.red * 2u
+                                                : (uint32_t)a.M * (uint32_t)a.ldx * 2u);
   // exact sizes: w[1] is W_up (GATED) or W_down from its row 16 on
   const uint32_t w_bytes = (uint32_t)a.R * (uint32_t)a.red * 2u;
   const buffer_rsrc rw[2] = {make_rsrc(a.w[0], w_bytes),
                              make_rsrc(a.w[1], GATED ? w_bytes : w_bytes - 16u * (uint32_t)a.red * 2u)};
 
-  i32x4 xf[DS_RD][8];
+  i32x4 xf[DS_RD][8 * MT];  // [stage in flight][MFMA step q][token tile]
 
   // Stage i_req of this wavefront's stream: token operands into xf[u], weights into ring slot u.
   auto issue_stage = [&](int i_req, int u) __attribute__((always_inline)) {
@@ -176,11 +203,13 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     int row0, valid;
     block_rows(j, row0, valid);
     uint32_t koff = (uint32_t)((c0 + c) * DS_CH) * 2u;
-    // token operand of the stage's q-th MFMA: 64 bytes further along each row of x, or the next
-    // 1 KiB fragment of H (a stage of 256 elements x 16 token slots is 8 KiB)
-    const uint32_t xstage = tiled_x ? koff * 16u : koff;
+    // token operand of the stage's q-th MFMA step: 64 bytes further along each row of x, or the
+    // next fragment of H (a stage of 256 elements x 16 MT token slots is 8 MT KiB)
+    const uint32_t xstage = tiled_x ? koff * (16u * MT) : koff;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) xf[u][q] = load16_async(rx, xoff, xstage + q * xq);
+    for (int q = 0; q < 8; ++q)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xf[u][q * MT + t] = load16_async(rx, xoff[t], xstage + q * xq);
     uint32_t slot = lds_base + (uint32_t)u * SLOT;
     uint32_t woffs = (uint32_t)row0 * (uint32_t)a.red * 2u + koff;
 #pragma unroll
@@ -192,9 +221,11 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     }
   };
 
-  f32x4v acc[NMAT];
+  f32x4v acc[NMAT][MT];
 #pragma unroll
-  for (int m = 0; m < NMAT; ++m) acc[m] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[m][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
   for (int p = 0; p < DS_RD; ++p) issue_stage(p, p);
@@ -205,75 +236,87 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     for (int u = 0; u < DS_RD; ++u) {
       const int i = i0 + u;
       if (i < total) {
-        wait_vmem_keep<(DS_RD - 1) * LPS>(xf[u]);
+        wait_vmem_keep<YOUNGER, 8 * MT>(xf[u]);
         const char* slot = ring + u * SLOT;
 #pragma unroll
         for (int ks = 0; ks < DS_CH / 32; ++ks) {
           int pos = ((ks * 4 + kg) ^ r16) << 4;
-          vec8 xv = __builtin_bit_cast(vec8, xf[u][ks]);
 #pragma unroll
           for (int m = 0; m < NMAT; ++m) {
             vec8 wf = *(const vec8*)(slot + m * DS_REGION + r16 * 512 + pos);
-            acc[m] = Mfma16x<T>::run(wf, xv, acc[m]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+              acc[m][t] = Mfma16x<T>::run(wf, __builtin_bit_cast(vec8, xf[u][ks * MT + t]), acc[m][t]);
           }
         }
         // The MFMAs above consumed every LDS read of this slot, so it can be refilled.
         issue_stage(i + DS_RD, u);
 
         if (++in_block == spb) {
-          // Block finished: wavefronts 1.. hand their partial sums to wavefront 0.  A lane holds
-          // token row m = lane%16 and, per region, weight rows 4*(lane/16) + r of the block.
+          // Block finished: wavefronts 1.. hand their partial sums to wavefront 0.  A lane holds,
+          // per token tile t, token row 16 t + lane%16 and, per region, weight rows 4*(lane/16) + r
+          // of the block.
           in_block = 0;
-          float* pp = part + (blk & 1) * ((DS_WAVES - 1) * NMAT * 256);
+          float* pp = part + (blk & 1) * ((DS_WAVES - 1) * NMAT * MT * 256);
           if (wave > 0) {
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
-              *(f32x4v*)(pp + ((wave - 1) * NMAT + m) * 256 + lane * 4) = acc[m];
+#pragma unroll
+              for (int t = 0; t < MT; ++t)
+                *(f32x4v*)(pp + (((wave - 1) * NMAT + m) * MT + t) * 256 + lane * 4) = acc[m][t];
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
           __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-          if (wave == 0 && ((GATED && a.tiled) || r16 < a.M)) {
+          if (wave == 0) {
             int row0, valid;
             block_rows(blk, row0, valid);
             const int r0 = row0 + 4 * kg;  // this lane's four rows (of each region)
-            float v[NMAT][4];
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m) {
+            for (int t = 0; t < MT; ++t) {
+              const int tok = 16 * t + r16;
+              if (!((GATED && a.tiled) || tok < a.M)) continue;
+              float v[NMAT][4];
 #pragma unroll
-              for (int r = 0; r < 4; ++r) v[m][r] = acc[m][r];
+              for (int m = 0; m < NMAT; ++m) {
 #pragma unroll
-              for (int w = 0; w < DS_WAVES - 1; ++w) {
-                f32x4v o = *(const f32x4v*)(pp + (w * NMAT + m) * 256 + lane * 4);
+                for (int r = 0; r < 4; ++r) v[m][r] = acc[m][t][r];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) v[m][r] += o[r];
+                for (int w = 0; w < DS_WAVES - 1; ++w) {
+                  f32x4v o = *(const f32x4v*)(pp + ((w * NMAT + m) * MT + t) * 256 + lane * 4);
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) v[m][r] += o[r];
+                }
+                if (a.bias[m] && 4 * kg + (GATED ? 0 : 16 * m) < valid)
+                  add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
               }
-              if (a.bias[m] && 4 * kg + (GATED ? 0 : 16 * m) < valid)
-                add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
-            }
-            if (GATED) {
-              float res[4];
-              act_fwd_w<4>(a.act, v[0], res);
+              if (GATED) {
+                float res[4];
+                act_fwd_w<4>(a.act, v[0], res);
 #pragma unroll
-              for (int r = 0; r < 4; ++r) res[r] *= v[NMAT - 1][r];
-              // Fragment order: H goes out the way the down projection's MFMAs take it in,
-              // [N/8][16 token slots][8 elements], so that a token-operand fragment there is one
-              // contiguous KiB instead of 16 row pieces of 64 bytes.  All 16 slots are written
-              // (slots past M repeat the last token), so nothing uninitialised is multiplied.
-              if (4 * kg < valid) {
-                if (a.tiled)
-                  store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * 16 + r16) * 8 + (r0 & 7), res);
-                else
-                  store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0, res);
+                for (int r = 0; r < 4; ++r) res[r] *= v[NMAT - 1][r];
+                // Fragment order: H goes out the way the down projection's MFMAs take it in,
+                // [N/8][16 MT token slots][8 elements], so that a token-operand fragment there is
+                // 4 runs of 256 MT bytes (one contiguous KiB for MT = 1) instead of 16 row pieces of
+                // 64 bytes.  All slots are written (slots past M repeat the last token), so nothing
+                // uninitialised is multiplied.
+                if (4 * kg < valid) {
+                  if (a.tiled)
+                    store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * (16 * MT) + tok) * 8 + (r0 & 7), res);
+                  else
+                    store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + r0, res);
+                }
+              } else {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+                  if (4 * kg + 16 * m < valid) store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + r0 + 16 * m, v[m]);
               }
-            } else {
-#pragma unroll
-              for (int m = 0; m < NMAT; ++m)
-                if (4 * kg + 16 * m < valid) store_w<T, 4>((T*)a.out + (size_t)r16 * a.ldo + r0 + 16 * m, v[m]);
             }
           }
 #pragma unroll
-          for (int m = 0; m < NMAT; ++m) acc[m] = f32x4v{0.f, 0.f, 0.f, 0.f};
+          for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[m][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
           ++blk;
         }
       }
@@ -282,10 +325,11 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   wait_vmem<0>();
 }
 
-template <typename T, bool GATED, int NMAT>
+template <typename T, bool GATED, int NMAT, int MT>
 static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
-  constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT) * NMAT * DS_REGION + 2 * (DS_WAVES - 1) * NMAT * 256 * 4;
-  auto kern = decode_stream_kernel<T, GATED, NMAT>;
+  constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT, MT) * NMAT * DS_REGION + 2 * (DS_WAVES - 1) * NMAT * MT * 256 * 4;
+  static_assert(LDS <= 160 * 1024, "a workgroup has 160 KiB of LDS");
+  auto kern = decode_stream_kernel<T, GATED, NMAT, MT>;
   static LdsAttrOnce lds_attr;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
   // one workgroup per CU, each with its share of the rows; fewer when that would be under 16 rows
@@ -296,11 +340,11 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
 
 // Layout of the intermediate H between the two kernels.  Row-major [M, N] costs the down projection
 // M pieces of 64 bytes per token-operand fragment, fragment order always one KiB (16 token slots):
-// cheaper from about half-full upwards.
+// cheaper from about half-full upwards.  Two token tiles always use fragment order.
 static int ds_h_tiled(int M) { return M > GMLP_DECODE_TILED_MIN ? 1 : 0; }
 
 bool decode_stream_supported(int M, int K, int N) {
-  return M >= 1 && M <= 16 && K % DS_CH == 0 && N % DS_CH == 0 && K >= DS_WAVES * DS_CH && N >= DS_WAVES * DS_CH &&
+  return M >= 1 && M <= 32 && K % DS_CH == 0 && N % DS_CH == 0 && K >= DS_WAVES * DS_CH && N >= DS_WAVES * DS_CH &&
          (int64_t)K * N * 2 < ((int64_t)1 << 31);
 }
 
@@ -314,12 +358,15 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
   if (num_cu <= 0) num_cu = 256;
   const int tiled = ds_h_tiled(M);
   StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act, tiled};
-  hipError_t e = launch_stream<T, true, 2>(a1, num_cu, s);
-  if (e != hipSuccess) return e;
   StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY, tiled};
   // 32-row blocks halve the L2 traffic for H; worth it when a CU's share of the rows exceeds 16
-  if (K > 16 * num_cu) return launch_stream<T, false, 2>(a2, num_cu, s);
-  return launch_stream<T, false, 1>(a2, num_cu, s);
+  const bool wide = K > 16 * num_cu;
+  if (M <= 16) {
+    if (hipError_t e = launch_stream<T, true, 2, 1>(a1, num_cu, s)) return e;
+    return wide ? launch_stream<T, false, 2, 1>(a2, num_cu, s) : launch_stream<T, false, 1, 1>(a2, num_cu, s);
+  }
+  if (hipError_t e = launch_stream<T, true, 2, 2>(a1, num_cu, s)) return e;
+  return wide ? launch_stream<T, false, 2, 2>(a2, num_cu, s) : launch_stream<T, false, 1, 2>(a2, num_cu, s);
 }
 
 template hipError_t launch_decode_stream<f16>(const f16*, const f16*, const f16*, const f16*,

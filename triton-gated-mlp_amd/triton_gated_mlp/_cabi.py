@@ -16,7 +16,7 @@ from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD, GMLP_OP_GATEUP_FWD = 0, 1, 2, 3, 4
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
 # tables (src/triton_gated_mlp/gated_mlp.py:17-37).

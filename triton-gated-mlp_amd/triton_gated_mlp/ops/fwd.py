@@ -127,7 +127,8 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
     return out
 
 
-DECODE_MAX_M = 16
+DECODE_MAX_M = 32
+DECODE_PREFERRED_MAX_M = 20
 
 
 def max_rows_32bit(K: int, N: int, dtype: torch.dtype) -> Optional[int]:
@@ -145,8 +146,15 @@ def max_rows_32bit(K: int, N: int, dtype: torch.dtype) -> Optional[int]:
     return max(256, (limit - 1) // (2 * width) // 256 * 256)
 
 
+def _decode_streams(K: int, N: int) -> bool:
+    """Shapes the LDS-ring streaming kernels take (the others run on plainer skinny-M kernels)."""
+    return K % 256 == 0 and N % 256 == 0 and K >= 768 and N >= 768 and K * N < (1 << 30)
+
+
 def decode_supported(M: int, K: int, N: int, dtype: torch.dtype = torch.float16) -> bool:
-    return dtype in (torch.float16, torch.bfloat16) and 1 <= M <= DECODE_MAX_M and K % 32 == 0 and N % 256 == 0
+    if dtype not in (torch.float16, torch.bfloat16) or K % 32 != 0 or N % 256 != 0:
+        return False
+    return 1 <= M <= 16 or (16 < M <= DECODE_MAX_M and _decode_streams(K, N))
 
 
 def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16, num_cu: int = 256) -> bool:
@@ -156,9 +164,12 @@ def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16,
     W_gate/W_up, and of 32 or 16 rows of W_down), so they need widths that give each unit at least
     a block of W_gate/W_up rows and half a block of W_down rows; from there they beat or match the
     general path (GEMMs with split reductions) for every M <= 16 (measured on MI355X at the widths
-    of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384 and 2048 x 8192).
+    of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384 and 2048 x 8192).  With two token tiles
+    (16 < M <= 32) the token operands cost as much L2 traffic as the weights cost HBM traffic: the
+    kernels still win by 4 to 11 % at M = 17 and draw level between M = 24 and 32, so the module
+    takes them up to M = 20.
     """
-    return decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu and K >= 8 * num_cu
+    return M <= DECODE_PREFERRED_MAX_M and decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu and K >= 8 * num_cu
 
 
 def decode_fwd(
@@ -171,7 +182,7 @@ def decode_fwd(
     b_down: Optional[Tensor],
     act_fn: str = "silu",
 ) -> Tensor:
-    """Whole-MLP forward for M <= 16 token rows: every weight byte is read from HBM once."""
+    """Whole-MLP forward for M <= 32 token rows: every weight byte is read from HBM once."""
     validate_dimensions(x, W_up, b_up, W_gate, b_gate)
     M, K = x.shape
     N = W_up.shape[0]
@@ -182,7 +193,8 @@ def decode_fwd(
     act = _cabi.act_code(act_fn)
     x, W_gate, W_up, W_down = _c(x), _c(W_gate), _c(W_up), _c(W_down)
     b_gate, b_up, b_down = _c(b_gate), _c(b_up), _c(b_down)
-    h = torch.empty((16, N), dtype=x.dtype, device=dev)  # scratch: H for 16 token slots, library's layout
+    # scratch: H for 16 or 32 token slots, in the library's layout
+    h = torch.empty((16 if M <= 16 else 32, N), dtype=x.dtype, device=dev)
     y = torch.empty((M, K), dtype=x.dtype, device=dev)
     with torch.cuda.device(dev):
         _cabi.check(
