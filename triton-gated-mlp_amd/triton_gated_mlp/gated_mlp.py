@@ -131,6 +131,16 @@ class FusedGatedMLPFunction(Function):
         return grads[: len(need)]  # apply() may have been called with the 5 reference arguments only
 
 
+_CU_COUNT = {}
+
+
+def _compute_units(device: torch.device) -> int:
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _CU_COUNT:
+        _CU_COUNT[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _CU_COUNT[index]
+
+
 class FusedGatedMLPFullFunction(Function):
     """Whole MLP as one autograd node, so dY -> (dG, dU) is a single GEMM with a fused epilogue."""
 
@@ -265,13 +275,16 @@ class FusedGatedMLP(_GatedMLPBase):
                     for i in range(0, M, rows)
                 ]
             )
-        inference = not torch.is_grad_enabled() or not (
-            x2.requires_grad or any(q.requires_grad for q in self.parameters())
+        inference = not torch.is_grad_enabled() or not any(
+            t is not None and t.requires_grad for t in (x2, W_gate, b_gate, W_up, b_up, W_down, b_down)
         )
-        if inference and p == 0.0 and x2.is_cuda and _fwd.decode_preferred(
-            M, K, self.intermediate_size, x2.dtype, torch.cuda.get_device_properties(x2.device).multi_processor_count
-        ):
-            return _fwd.decode_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, self.act_fn)
+        if inference and p == 0.0 and x2.is_cuda:
+            # Nothing to differentiate: no autograd node (its bookkeeping costs more host time than a
+            # short batch's kernels take to enqueue), and the weight-streaming kernels for skinny M.
+            if _fwd.decode_preferred(M, K, self.intermediate_size, x2.dtype, _compute_units(x2.device)):
+                return _fwd.decode_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, self.act_fn)
+            hs = _fwd.gateup_fwd(x2, W_gate, b_gate, W_up, b_up, 0.0, 0, 0, save_activations=False, act_fn=self.act_fn)
+            return _fwd.linear_fwd(hs.hidden, W_down, b_down)
         seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
         return FusedGatedMLPFullFunction.apply(
             x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p, seed, offset, self.recompute_activations, self.act_fn
