@@ -262,3 +262,44 @@ def test_decode_preferred_needs_widths_that_fill_the_chip():
     assert not decode_preferred(1, 1024, 2048)  # fewer W_gate/W_up blocks than compute units
     assert not decode_preferred(1, 1024, 8192)  # a quarter of a W_down block per compute unit
     assert not decode_preferred(1, 8192, 28672, torch.float32)
+
+
+def test_async_load_checker_flags_registers_touched_before_their_wait(tmp_path):
+    """The build-time check of the streaming kernels' assembly: a load's destination registers may
+    not be named by any instruction before the s_waitcnt that covers the load (in-order return: a
+    wait for N leaves only the N youngest loads in flight; loads into LDS have no destination)."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location(
+        "check_async_loads", ROOT / "triton-gated-mlp_amd" / "csrc" / "check_async_loads.py"
+    )
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+
+    good = tmp_path / "good.s"
+    good.write_text(
+        "_Z4kernv:\n"
+        "\tbuffer_load_dwordx4 v[4:7], v1, s[0:3], s8 offen\n"
+        "\tbuffer_load_dwordx4 v2, s[0:3], s8 offen lds\n"
+        "\tbuffer_load_dwordx4 v[8:11], v1, s[0:3], s9 offen\n"
+        "\tv_add_u32_e32 v1, 16, v1\n"            # the address register is free to change
+        "\ts_waitcnt vmcnt(1)\n"                   # retires the first two loads
+        "\tv_accvgpr_write_b32 a0, v4\n"
+        "\ts_waitcnt vmcnt(0)\n"
+        "\tv_mfma_f32_16x16x32_f16 a[0:3], v[4:7], v[8:11], a[0:3]\n"
+        "\ts_endpgm\n"
+    )
+    assert mod.check(str(good)) == 0
+    bad = tmp_path / "bad.s"
+    bad.write_text(
+        "_Z4kernv:\n"
+        "\tbuffer_load_dwordx4 v[4:7], v1, s[0:3], s8 offen\n"
+        "\tbuffer_load_dwordx4 v[8:11], v1, s[0:3], s9 offen\n"
+        "\ts_waitcnt vmcnt(1)\n"
+        "\tv_accvgpr_write_b32 a1, v9\n"           # the second load is still in flight
+        "\ts_waitcnt vmcnt(0)\n"
+        "\ts_endpgm\n"
+        "_Z5kern2v:\n"
+        "\ts_endpgm\n"
+    )
+    assert mod.check(str(bad)) == 1
