@@ -29,6 +29,11 @@ struct GemmArgs {
   int splits;        // pipelined kernel with a split-reduction epilogue only: number of workgroups
                      // that share one output tile, each reducing a contiguous range of 64-wide
                      // reduction tiles into a partial result of its own (0 or 1: no split)
+  int rotate;        // pipelined kernel: workgroup u starts its reduction range at tile u mod length
+                     // and wraps around.  For problems whose workgroups share no weight rows (one
+                     // row of output tiles): they would otherwise all read the same offset along
+                     // their rows at the same time, which for the usual power-of-two row pitches
+                     // crowds onto a few memory channels.
 };
 
 // Workgroup id -> output tile.  The hardware deals consecutive workgroup ids round-robin to the
@@ -322,6 +327,29 @@ struct EpiStore {
                                                const Prefetch<W>&) {
     apply<W>(a, m, n, v, w);
   }
+  // Accumulator-layout interface: the arithmetic runs on 4 consecutive columns of one row, as an
+  // MFMA leaves them in a lane, and yields the output planes already rounded to T; the kernel then
+  // transposes 2-byte elements through LDS instead of 4-byte ones.  Same operations per element
+  // as apply(), so the results are bit-identical.  Everything that would branch (optional biases,
+  // optional outputs) stays out of the way of the accumulators: biases arrive as values (zeros
+  // when absent), optional outputs are whole planes that a uniform branch skips.
+  static constexpr bool PACKED = true;
+  static constexpr int PLANES = 1;
+  static constexpr int NBIAS = 1;
+  static constexpr bool STREAM_OUT = true;
+  static __device__ __forceinline__ int planes_on(const Args&) { return 1; }
+  static __device__ __forceinline__ T* plane(const Args& a, int) { return a.out; }
+  static __device__ __forceinline__ void bias4(const Args& a, int n, float (&b)[NBIAS][4]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) b[0][r] = 0.f;
+    if (a.bias) load_w<T, 4>(a.bias + n, b[0]);
+  }
+  static __device__ __forceinline__ void pack4(const Args&, int, int, const float (&b)[NBIAS][4],
+                                               const float* v, const float*,
+                                               typename PackW<T, 4>::type (&o)[PLANES]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[0][r] = Traits<T>::from_f32(v[r] + b[0][r]);
+  }
 };
 
 // Split reduction: workgroup `split` of an output tile stores its fp32 partial sums to
@@ -338,6 +366,7 @@ struct EpiPartial {
   static constexpr int PREFETCH_DEPTH = 0;
   static constexpr bool HAS_ACT = false;
   static constexpr bool SPLIT = true;
+  static constexpr bool PACKED = false;
   template <int W>
   struct Prefetch {};
   template <int W>
@@ -415,6 +444,58 @@ struct EpiGateUp {
                                                const Prefetch<W>&) {
     apply<W, ACT>(a, m, n, g, u);
   }
+  static constexpr bool PACKED = false;  // see EpiGateUpPacked
+};
+
+// The same epilogue for kernels that run it in the accumulator layout (see EpiStore): SiLU, no
+// keep-mask output, G and U kept both or not at all (packed_eligible; the launcher picks the
+// kernel).  Planes H, G, U; the optional parts are uniform branches around small pieces of
+// straight-line code.
+template <typename T>
+struct EpiGateUpPacked : EpiGateUp<T> {
+  typedef typename EpiGateUp<T>::Args Args;
+  static constexpr bool PACKED = true;
+  static constexpr int PLANES = 3;
+  static constexpr int NBIAS = 2;
+  static constexpr bool STREAM_OUT = false;
+  static bool packed_eligible(const Args& a) {
+    return a.mask_out == nullptr && a.act == ACT_SILU && (a.g_save == nullptr) == (a.u_save == nullptr);
+  }
+  static __device__ __forceinline__ int planes_on(const Args& a) { return a.g_save != nullptr ? 3 : 1; }
+  static __device__ __forceinline__ T* plane(const Args& a, int p) {
+    return p == 0 ? a.h : p == 1 ? a.g_save : a.u_save;
+  }
+  static __device__ __forceinline__ void bias4(const Args& a, int n, float (&b)[NBIAS][4]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) b[0][r] = b[1][r] = 0.f;
+    if (a.b_gate) load_w<T, 4>(a.b_gate + n, b[0]);
+    if (a.b_up) load_w<T, 4>(a.b_up + n, b[1]);
+  }
+  static __device__ __forceinline__ void pack4(const Args& a, int m, int n, const float (&b)[NBIAS][4],
+                                               const float* gacc, const float* uacc,
+                                               typename PackW<T, 4>::type (&o)[PLANES]) {
+    float g[4], u[4], h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      g[r] = gacc[r] + b[0][r];
+      u[r] = uacc[r] + b[1][r];
+    }
+    act_fwd_w<4, ACT_SILU>(ACT_SILU, g, h);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] *= u[r];
+    if (a.drop.enabled) {
+      bool keep[4];
+      keep_w<4>(a.drop, (size_t)m * a.ldc + n, keep);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      o[0][r] = Traits<T>::from_f32(h[r]);
+      o[1][r] = Traits<T>::from_f32(g[r]);
+      o[2][r] = Traits<T>::from_f32(u[r]);
+    }
+  }
 };
 
 // Gating backward on W consecutive elements: dA = dH*keep/(1-p); dU = dA*act(G); dG = dA*U*act'(G)
@@ -479,6 +560,7 @@ struct EpiDh {
   }
   static constexpr bool HAS_ACT = true;
   static constexpr bool SPLIT = false;
+  static constexpr bool PACKED = false;  // G and U arrive row-wise: the arithmetic stays behind the transpose
   template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*,
                                                const Prefetch<W>& p) {

@@ -32,6 +32,11 @@ typedef bf16 DT;
 template <>
 hipError_t launch_gateup<DT>(int tile_class, const GemmArgs& ga, const EpiGateUp<DT>::Args& ea,
                              hipStream_t s) {
+  // the usual case (SiLU, no keep-mask output) has kernels of its own, see EpiGateUpPacked
+  if (EpiGateUpPacked<DT>::packed_eligible(ea)) {
+    if (tile_class == TILE_LARGE) return GMLP_LARGE(false, false, 2, EpiGateUpPacked, 128)(ga, ea, s);
+    if (tile_class == TILE_MEDIUM_FULL) return GMLP_MEDIUM(false, false, 2, EpiGateUpPacked, 64)(ga, ea, s);
+  }
   GMLP_DISPATCH(false, false, 2, EpiGateUp, 128, 64)
 }
 template <>

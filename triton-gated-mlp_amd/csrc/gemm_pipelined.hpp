@@ -3,8 +3,8 @@
 // Same contract as gemm_kernel (gemm.hpp): C[M,N] = sum_s sum_k A_s[m,k] * B_s[n,k], operands
 // reduction-contiguous (KC) or reduction-strided (KS), NB accumulator sets, fused epilogue.
 // Reduction tiles of 64 elements travel global -> LDS without passing through registers
-// (gemm_tiles.hpp) into a two-slot ring; the epilogue transposes accumulators through LDS so that
-// every global access is a 16-byte, row-contiguous one.
+// (gemm_tiles.hpp) into a two-slot ring; the epilogue transposes accumulators (or finished
+// results) through LDS so that every global access is a 16-byte, row-contiguous one.
 //
 // Ragged edges cost nothing in the main loop: operands are read through buffer descriptors of
 // their exact size, so whatever a tile addresses beyond the END of an operand reads as zero.
@@ -142,6 +142,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
     kt_first = split * per;
     kt_total = kt_first + per < kt_total ? kt_first + per : kt_total;
   }
+  // Order in which the range is read from memory (the sum does not mind): see GemmArgs::rotate.
+  const int kt_len = kt_total - kt_first;
+  const int rot = ga.rotate && kt_len > 0 ? u % kt_len : 0;
 
   // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
   // Buffer addressing uses 32-bit byte offsets from each operand's base; the host checks sizes.
@@ -190,6 +193,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // nobody reads again.
   auto issue_one = [&](int kt_req, int x) __attribute__((always_inline)) {
     int kt = kt_req < kt_total ? kt_req : kt_total - 1;
+    kt += rot;
+    kt = kt >= kt_total ? kt - kt_len : kt;
     int seg = kt >= kt_seg ? 1 : 0;
     int kk = kt - seg * kt_seg;
     buffer_rsrc r;
@@ -333,8 +338,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   tile_body(kt, std::false_type{});
   wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
 
-  // ---- epilogue: transpose MI-row slabs of the accumulators through LDS (fp32), then each lane
-  // owns 8 consecutive columns of one row.
+  // ---- epilogue: transpose MI-row slabs through LDS, after which each lane owns 8 consecutive
+  // columns of one row: the fp32 accumulators themselves, with the arithmetic behind the transpose
+  // (slabs), or, where the epilogue offers it, the finished 16-bit results (further down).
   __syncthreads();  // all wavefronts are done reading operand tiles
   constexpr int ELD = Cfg::EPI_LD;
   float* stg = (float*)(smem + wave * Cfg::EPI_WAVE_BYTES);
@@ -382,6 +388,72 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
       }
     }
   };
+  // Epilogues that offer it run their arithmetic in the accumulator layout (a lane holds 4
+  // consecutive columns of one row per 16x16 block) and hand over results already rounded to T:
+  // the transpose through LDS then moves 2-byte elements, one plane per output tensor.  The loop
+  // over the accumulators is one piece of straight-line code (alternatives that read the
+  // accumulators in several branches made the compiler copy all of them to VGPRs first).
+  // Staging of a wavefront: planes x [16 rows][WTN elements], row r's 8-byte unit u stored at
+  // u ^ 2 (r >> SH): the 32 lanes of a half-wave write (16 rows x 2 units) hit 64 distinct banks,
+  // and a 16-byte read of chunk c of row r finds it at c ^ (r >> SH), 16 lanes covering all banks.
+  if constexpr (MI == 16 && Epi::PACKED) {
+    typedef typename PackW<T, 4>::type vec4;
+    constexpr int P = Epi::PLANES;
+    constexpr int UPR = WTN / 4;                       // 8-byte units per staging row
+    constexpr int SH = UPR >= 32 ? 0 : (UPR == 16 ? 1 : 2);
+    static_assert(UPR == 32 || UPR == 16 || UPR == 8, "wavefront tiles are 32 to 128 columns wide");
+    static_assert(P * MI * WTN * 2 <= Cfg::EPI_WAVE_BYTES, "staging planes must fit the wavefront's share");
+    char* stp = smem + wave * Cfg::EPI_WAVE_BYTES;
+    const int cq = lane / MI;                          // which 4 columns of a 16-column block
+    const int planes_on = Epi::planes_on(ea);          // uniform
+    // biases of this lane's columns (zeros when there is none); columns past the edge read the
+    // last valid group instead and are dropped when it comes to storing
+    float bias[TN][Epi::NBIAS][4];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) Epi::bias4(ea, min(n0 + wn * WTN + j * MI + 4 * cq, ga.N - 4), bias[j]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m0 + wm * WTM + i * MI + mrow;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * WTN + j * MI + 4 * cq;
+        float v0[4], v1[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v0[r] = acc[j][i][r];
+          if constexpr (NB == 2) v1[r] = acc[TN + j][i][r];
+          else v1[r] = 0.f;
+        }
+        vec4 o[P];
+        Epi::pack4(ea, m, n, bias[j], v0, v1, o);
+        const int unit = (4 * j + cq) ^ (2 * (mrow >> SH));
+        *(vec4*)(stp + mrow * (WTN * 2) + unit * 8) = o[0];
+        if (P > 1 && planes_on > 1) {
+#pragma unroll
+          for (int pl = 1; pl < P; ++pl)
+            *(vec4*)(stp + pl * (MI * WTN * 2) + mrow * (WTN * 2) + unit * 8) = o[pl];
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        int row, m2, n2, cg;
+        item_pos(i * ITEMS + it, row, m2, n2, cg);
+        const int chunk = cg ^ (row >> SH);
+        const bool inside = m2 < ga.M && n2 < ga.N;
+#pragma unroll
+        for (int pl = 0; pl < P; ++pl) {
+          if (pl > 0 && planes_on <= 1) break;
+          vec8 val = *(const vec8*)(stp + pl * (MI * WTN * 2) + row * (WTN * 2) + chunk * 16);
+          if (inside) {
+            vec8* q = (vec8*)(Epi::plane(ea, pl) + (size_t)m2 * ea.ldc + n2);
+            if (Epi::STREAM_OUT) __builtin_nontemporal_store(val, q);
+            else *q = val;
+          }
+        }
+      }
+    }
+    return;
+  }
   if constexpr (Epi::HAS_ACT) {
     switch (ea.act) {
       case ACT_SILU: slabs(std::integral_constant<int, ACT_SILU>{}); break;
