@@ -203,7 +203,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
   GemmArgs ga = {};
   ga.A[0] = x; ga.A[1] = x; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
-  ga.nseg = 1; ga.group_m = pick_group(M, N, 2); ga.rotate = M <= 128;
+  ga.nseg = 1; ga.group_m = pick_group(M, N, 2); ga.rotate = M <= 512;
   int tc = pick_tile(dtype, M, N, K, 128);
   const int splits = pick_splits(dtype, M, N, K, (K + 63) / 64, 128);
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, N, 2);
@@ -241,7 +241,7 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   GemmArgs ga = {};
   ga.A[0] = a; ga.A[1] = a; ga.B[0] = w; ga.B[1] = w;
   ga.M = (int)M; ga.N = (int)C; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
-  ga.nseg = 1; ga.group_m = pick_group(M, C); ga.rotate = M <= 128;
+  ga.nseg = 1; ga.group_m = pick_group(M, C); ga.rotate = M <= 512;
   int tc = pick_tile(dtype, M, C, R, 256);
   const int splits = pick_splits(dtype, M, C, R, (R + 63) / 64);
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, C);
@@ -333,7 +333,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   GemmArgs ga = {};
   ga.A[0] = dg; ga.A[1] = du; ga.B[0] = w_gate; ga.B[1] = w_up;
   ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
-  ga.nseg = 2; ga.group_m = pick_group(M, K); ga.rotate = M <= 128;
+  ga.nseg = 2; ga.group_m = pick_group(M, K); ga.rotate = M <= 512;
   int tc = pick_tile(dtype, M, K, N, 256);
   const int splits = pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64));
   const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, K);

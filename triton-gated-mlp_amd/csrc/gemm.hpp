@@ -29,11 +29,13 @@ struct GemmArgs {
   int splits;        // pipelined kernel with a split-reduction epilogue only: number of workgroups
                      // that share one output tile, each reducing a contiguous range of 64-wide
                      // reduction tiles into a partial result of its own (0 or 1: no split)
-  int rotate;        // pipelined kernel: workgroup u starts its reduction range at tile u mod length
-                     // and wraps around.  For problems whose workgroups share no weight rows (one
-                     // row of output tiles): they would otherwise all read the same offset along
-                     // their rows at the same time, which for the usual power-of-two row pitches
-                     // crowds onto a few memory channels.
+  int rotate;        // pipelined kernel: the workgroups of tile column c start their reduction
+                     // range at tile c mod length and wrap around.  For short batches, which are
+                     // bound by streaming the B operand (the weights): the workgroups would
+                     // otherwise all read the same offset along their rows at the same time, which
+                     // for the usual power-of-two row pitches crowds onto a few memory channels.
+                     // Workgroups that share B rows keep the same order, so they still share them
+                     // in L2.
 };
 
 // Workgroup id -> output tile.  The hardware deals consecutive workgroup ids round-robin to the

@@ -144,7 +144,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   }
   // Order in which the range is read from memory (the sum does not mind): see GemmArgs::rotate.
   const int kt_len = kt_total - kt_first;
-  const int rot = ga.rotate && kt_len > 0 ? u % kt_len : 0;
+  const int rot = ga.rotate && kt_len > 0 ? tn_i % kt_len : 0;
 
   // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
   // Buffer addressing uses 32-bit byte offsets from each operand's base; the host checks sizes.
