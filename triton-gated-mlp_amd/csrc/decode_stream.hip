@@ -49,11 +49,21 @@ struct Mfma16x<bf16> {
 
 constexpr int DS_CH = 256;            // reduction elements per stage
 constexpr int DS_REGION = 16 * 512;   // bytes of one 16-row region
-// ring slots per wavefront (and stages in flight): 3 slots of two 16-row regions, or 4 of one
-// (3 with two token tiles: the token operands in flight are bounded by the registers, see below)
-constexpr int ds_ring_depth(int nmat, int mt) { return nmat == 2 || mt == 2 ? 3 : 4; }
+// ring slots per wavefront (and stages in flight): 3 slots of two matrices, or 4 of one (3 where
+// two token tiles go with 512-byte segments: the token operands in flight are bounded by the
+// registers, see the kernel)
+constexpr int ds_ring_depth(int nmat, int mt, int segb) { return nmat == 2 || (mt == 2 && segb == 512) ? 3 : 4; }
 constexpr int DS_WAVES = 3;           // wavefronts per workgroup
+// buffers for the partial sums that change hands at the end of a block: two (alternating) where
+// LDS holds them beside the rings, else one
+constexpr int ds_part_buffers(int nmat, int mt, int segb) {
+  return DS_WAVES * ds_ring_depth(nmat, mt, segb) * nmat * DS_REGION + 2 * (DS_WAVES - 1) * nmat * (512 / segb) * mt * 1024 <=
+                 160 * 1024
+             ? 2
+             : 1;
+}
 constexpr uint32_t DS_NOWHERE = 0x80000000u;  // voffset beyond any operand (operands are < 2 GiB)
+constexpr int DS_WIDE_SEGMENT_MAX_M = 20;     // two token tiles: 512-byte row segments up to here, 256 beyond
 #ifndef GMLP_DECODE_TILED_MIN
 #define GMLP_DECODE_TILED_MIN 10
 #endif
@@ -99,32 +109,51 @@ __device__ __forceinline__ void wait_vmem_keep(i32x4 (&x)[NX]) {
                  : "memory");
 }
 
-// NMAT: 16-row regions per stage (GATED: W_gate and W_up; otherwise 1 or 2 runs of W_down rows).
-// MT: tiles of 16 token slots (M <= 16 * MT).
-template <typename T, bool GATED, int NMAT, int MT>
+// NMAT: weight matrices / runs of rows per stage (GATED: W_gate and W_up; otherwise 1 or 2 runs of
+//       W_down rows).
+// MT:   tiles of 16 token slots (M <= 16 * MT).
+// SEGB: bytes of a weight row per stage, 512 or 256.  A stage always moves 8 KiB per matrix: 16
+//       rows x 512 bytes, or 32 rows x 256 bytes as two 16-row regions.  The second form halves
+//       the token operands fetched per weight byte (a stage spans half the reduction elements for
+//       twice the rows), which is what two token tiles need: with 16-row blocks their token
+//       operands cost as much L2 traffic as the weights cost HBM traffic.
+template <typename T, bool GATED, int NMAT, int MT, int SEGB>
 __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs a) {
   typedef typename Traits<T>::vec8 vec8;
   static_assert(NMAT == 2 || (NMAT == 1 && !GATED), "gated blocks stream two matrices");
-  constexpr int DS_RD = ds_ring_depth(NMAT, MT);
+  static_assert(SEGB == 512 || SEGB == 256, "row segment of a stage");
+  constexpr int DS_RD = ds_ring_depth(NMAT, MT, SEGB);
+  constexpr int HALVES = 512 / SEGB;          // 16-row regions per matrix and stage
+  constexpr int NREG = NMAT * HALVES;         // 16-row regions per stage
+  constexpr int REGION = 16 * SEGB;           // bytes of a region
+  constexpr int CH = SEGB / 2;                // reduction elements per stage
+  constexpr int KS = CH / 32;                 // MFMA steps per stage
+  constexpr int CPR = SEGB / 16;              // 16-byte chunks per row segment
+  constexpr int LPR = REGION / 1024;          // load instructions per region (64 lanes x 16 bytes each)
   // The token operands in flight live in VGPRs that the loads fill asynchronously.  Were there not
   // enough of the 256 left beside them, the compiler would park them elsewhere right after the
   // load instruction, before the data has arrived.
-  static_assert(DS_RD * 8 * MT * 4 <= 192, "token operands in flight must leave room in the VGPRs");
-  constexpr int BLOCK_ROWS = GATED ? 16 : 16 * NMAT;  // weight rows (per matrix) a block advances by
-  constexpr int SLOT = NMAT * DS_REGION;
-  constexpr int LPS = 8 * MT + 8 * NMAT;  // load instructions per stage (token operands + weights)
+  static_assert(DS_RD * KS * MT * 4 <= 192, "token operands in flight must leave room in the VGPRs");
+  // weight rows (per matrix) a block advances by
+  constexpr int BLOCK_ROWS = GATED ? 16 * HALVES : 16 * NREG;
+  constexpr int SLOT = NREG * REGION;
+  constexpr int LPS = KS * MT + NREG * LPR;  // load instructions per stage (token operands + weights)
   // A stage is complete when no more than the DS_RD - 1 younger stages are in flight.  vmcnt has 6
   // bits: where that count exceeds 63 the wait also covers the first token-operand loads of the
   // next stage (issued right behind the awaited weights, and loads return in order).
   constexpr int YOUNGER = (DS_RD - 1) * LPS < 63 ? (DS_RD - 1) * LPS : 63;
-  static_assert((DS_RD - 1) * LPS - YOUNGER <= 8 * MT, "the wait may only reach into the next stage's token operands");
+  static_assert((DS_RD - 1) * LPS - YOUNGER <= KS * MT, "the wait may only reach into the next stage's token operands");
+  // Partial sums change hands through LDS in two alternating buffers, or, where LDS does not hold
+  // two, in one buffer with a second barrier behind its readers.
+  constexpr int PART_FLOATS = (DS_WAVES - 1) * NREG * MT * 256;
+  constexpr int PARITIES = ds_part_buffers(NMAT, MT, SEGB);
 
   extern __shared__ __align__(1024) char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem + wave * (DS_RD * SLOT);
   char* ring = smem + wave * (DS_RD * SLOT);
-  float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [2 parities][waves-1][NMAT][MT][64][4]
+  float* part = (float*)(smem + DS_WAVES * DS_RD * SLOT);  // [parities][waves-1][NREG][MT][64][4]
 
   // Blocks of BLOCK_ROWS weight rows go round-robin over the workgroups (block b, b + G, ...: at any
   // time the chip streams one contiguous band of rows) for as many rounds as every workgroup gets a
@@ -148,7 +177,7 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
       valid = t_end - row0;
     }
   };
-  const int chunks = a.red / DS_CH;
+  const int chunks = a.red / CH;
   // wavefront w reduces chunks [c0, c0 + spb)
   const int c0 = (chunks * wave) / DS_WAVES;
   const int spb = (chunks * (wave + 1)) / DS_WAVES - c0;
@@ -160,14 +189,14 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   // hidden sizes) those addresses crowd onto a few memory channels: 154 -> 142 us at K = 8192.
   const int rot = (int)blockIdx.x % spb;
 
-  // Per-lane byte offsets: weights, 8 load instructions per region (2 rows x 512 bytes each);
+  // Per-lane byte offsets: weights, LPR load instructions per region (1024 / SEGB rows each);
   // token operands, the 16 bytes of token row 16 t + lane%16 this lane feeds to the MFMAs of tile t.
   const int r16 = lane & 15, kg = lane >> 4;
-  uint32_t woff[8], xoff[MT];
-  int wrow[8];  // row of the region that load q of this lane fetches
+  uint32_t woff[LPR], xoff[MT];
+  int wrow[LPR];  // row of the region that load q of this lane fetches
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    int row = 2 * q + (lane >> 5), pos = lane & 31;
+  for (int q = 0; q < LPR; ++q) {
+    int row = (64 / CPR) * q + lane / CPR, pos = lane % CPR;
     wrow[q] = row;
     woff[q] = (uint32_t)(row * a.red + (pos ^ row) * 8) * 2u;
   }
@@ -187,12 +216,13 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   // exact size: an offset past the end reads as zero instead of touching memory
   const buffer_rsrc rx = make_rsrc(a.x, tiled_x ? (uint32_t)(16 * MT) * (uint32_t)a.red * 2u
                                                 : (uint32_t)a.M * (uint32_t)a.ldx * 2u);
-  // exact sizes: w[1] is W_up (GATED) or W_down from its row 16 on
-  const uint32_t w_bytes = (uint32_t)a.R * (uint32_t)a.red * 2u;
-  const buffer_rsrc rw[2] = {make_rsrc(a.w[0], w_bytes),
-                             make_rsrc(a.w[1], GATED ? w_bytes : w_bytes - 16u * (uint32_t)a.red * 2u)};
+  // exact sizes; region g of a stage: GATED: matrix g / HALVES, rows 16 (g % HALVES) .. +15 of the
+  // block; otherwise rows 16 g .. +15 of the block of W_down
+  const uint32_t pitch = (uint32_t)a.red * 2u;
+  const uint32_t w_bytes = (uint32_t)a.R * pitch;
+  const buffer_rsrc rw[2] = {make_rsrc(a.w[0], w_bytes), make_rsrc(GATED ? a.w[1] : a.w[0], w_bytes)};
 
-  i32x4 xf[DS_RD][8 * MT];  // [stage in flight][MFMA step q][token tile]
+  i32x4 xf[DS_RD][KS * MT];  // [stage in flight][MFMA step q][token tile]
 
   // Stage i_req of this wavefront's stream: token operands into xf[u], weights into ring slot u.
   auto issue_stage = [&](int i_req, int u) __attribute__((always_inline)) {
@@ -202,30 +232,32 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     c = c < spb ? c : c - spb;
     int row0, valid;
     block_rows(j, row0, valid);
-    uint32_t koff = (uint32_t)((c0 + c) * DS_CH) * 2u;
+    uint32_t koff = (uint32_t)((c0 + c) * CH) * 2u;
     // token operand of the stage's q-th MFMA step: 64 bytes further along each row of x, or the
-    // next fragment of H (a stage of 256 elements x 16 MT token slots is 8 MT KiB)
+    // next fragment of H (a stage of CH elements x 16 MT token slots)
     const uint32_t xstage = tiled_x ? koff * (16u * MT) : koff;
 #pragma unroll
-    for (int q = 0; q < 8; ++q)
+    for (int q = 0; q < KS; ++q)
 #pragma unroll
       for (int t = 0; t < MT; ++t) xf[u][q * MT + t] = load16_async(rx, xoff[t], xstage + q * xq);
     uint32_t slot = lds_base + (uint32_t)u * SLOT;
-    uint32_t woffs = (uint32_t)row0 * (uint32_t)a.red * 2u + koff;
+    uint32_t woffs = (uint32_t)row0 * pitch + koff;
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) {
-      const int valid_m = GATED ? valid : valid - 16 * m;
+    for (int g = 0; g < NREG; ++g) {
+      const int first = GATED ? 16 * (g % HALVES) : 16 * g;  // region's first row within the block
+      const int valid_g = valid - first;
 #pragma unroll
-      for (int q = 0; q < 8; ++q)
-        load16_to_lds<true>(rw[m], wrow[q] < valid_m ? woff[q] : DS_NOWHERE, woffs, slot + m * DS_REGION + q * 1024);
+      for (int q = 0; q < LPR; ++q)
+        load16_to_lds<true>(rw[GATED ? g / HALVES : 0], wrow[q] < valid_g ? woff[q] : DS_NOWHERE,
+                            woffs + (uint32_t)first * pitch, slot + g * REGION + q * 1024);
     }
   };
 
-  f32x4v acc[NMAT][MT];
+  f32x4v acc[NREG][MT];
 #pragma unroll
-  for (int m = 0; m < NMAT; ++m)
+  for (int g = 0; g < NREG; ++g)
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[m][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < MT; ++t) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
   for (int p = 0; p < DS_RD; ++p) issue_stage(p, p);
@@ -236,17 +268,17 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
     for (int u = 0; u < DS_RD; ++u) {
       const int i = i0 + u;
       if (i < total) {
-        wait_vmem_keep<YOUNGER, 8 * MT>(xf[u]);
+        wait_vmem_keep<YOUNGER, KS * MT>(xf[u]);
         const char* slot = ring + u * SLOT;
 #pragma unroll
-        for (int ks = 0; ks < DS_CH / 32; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
           int pos = ((ks * 4 + kg) ^ r16) << 4;
 #pragma unroll
-          for (int m = 0; m < NMAT; ++m) {
-            vec8 wf = *(const vec8*)(slot + m * DS_REGION + r16 * 512 + pos);
+          for (int g = 0; g < NREG; ++g) {
+            vec8 wf = *(const vec8*)(slot + g * REGION + r16 * SEGB + pos);
 #pragma unroll
             for (int t = 0; t < MT; ++t)
-              acc[m][t] = Mfma16x<T>::run(wf, __builtin_bit_cast(vec8, xf[u][ks * MT + t]), acc[m][t]);
+              acc[g][t] = Mfma16x<T>::run(wf, __builtin_bit_cast(vec8, xf[u][ks * MT + t]), acc[g][t]);
           }
         }
         // The MFMAs above consumed every LDS read of this slot, so it can be refilled.
@@ -255,15 +287,15 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
         if (++in_block == spb) {
           // Block finished: wavefronts 1.. hand their partial sums to wavefront 0.  A lane holds,
           // per token tile t, token row 16 t + lane%16 and, per region, weight rows 4*(lane/16) + r
-          // of the block.
+          // of the region.
           in_block = 0;
-          float* pp = part + (blk & 1) * ((DS_WAVES - 1) * NMAT * MT * 256);
+          float* pp = part + (PARITIES == 2 ? (blk & 1) * PART_FLOATS : 0);
           if (wave > 0) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int g = 0; g < NREG; ++g)
 #pragma unroll
               for (int t = 0; t < MT; ++t)
-                *(f32x4v*)(pp + (((wave - 1) * NMAT + m) * MT + t) * 256 + lane * 4) = acc[m][t];
+                *(f32x4v*)(pp + (((wave - 1) * NREG + g) * MT + t) * 256 + lane * 4) = acc[g][t];
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
           __builtin_amdgcn_s_barrier();
@@ -271,52 +303,64 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
           if (wave == 0) {
             int row0, valid;
             block_rows(blk, row0, valid);
-            const int r0 = row0 + 4 * kg;  // this lane's four rows (of each region)
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
               const int tok = 16 * t + r16;
               if (!((GATED && a.tiled) || tok < a.M)) continue;
-              float v[NMAT][4];
+              float v[NREG][4];
 #pragma unroll
-              for (int m = 0; m < NMAT; ++m) {
+              for (int g = 0; g < NREG; ++g) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) v[m][r] = acc[m][t][r];
+                for (int r = 0; r < 4; ++r) v[g][r] = acc[g][t][r];
 #pragma unroll
                 for (int w = 0; w < DS_WAVES - 1; ++w) {
-                  f32x4v o = *(const f32x4v*)(pp + ((w * NMAT + m) * MT + t) * 256 + lane * 4);
+                  f32x4v o = *(const f32x4v*)(pp + ((w * NREG + g) * MT + t) * 256 + lane * 4);
 #pragma unroll
-                  for (int r = 0; r < 4; ++r) v[m][r] += o[r];
+                  for (int r = 0; r < 4; ++r) v[g][r] += o[r];
                 }
-                if (a.bias[m] && 4 * kg + (GATED ? 0 : 16 * m) < valid)
-                  add_w<T, 4>((const T*)a.bias[m] + r0 + (GATED ? 0 : 16 * m), v[m]);
+                // this lane's four rows of the region, as rows of the block
+                const int first = (GATED ? 16 * (g % HALVES) : 16 * g) + 4 * kg;
+                const T* bias = (const T*)a.bias[GATED ? g / HALVES : 0];
+                if (bias && first < valid) add_w<T, 4>(bias + row0 + first, v[g]);
               }
               if (GATED) {
-                float res[4];
-                act_fwd_w<4>(a.act, v[0], res);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) res[r] *= v[NMAT - 1][r];
-                // Fragment order: H goes out the way the down projection's MFMAs take it in,
-                // [N/8][16 MT token slots][8 elements], so that a token-operand fragment there is
-                // 4 runs of 256 MT bytes (one contiguous KiB for MT = 1) instead of 16 row pieces of
-                // 64 bytes.  All slots are written (slots past M repeat the last token), so nothing
-                // uninitialised is multiplied.
-                if (4 * kg < valid) {
-                  if (a.tiled)
-                    store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * (16 * MT) + tok) * 8 + (r0 & 7), res);
-                  else
-                    store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + r0, res);
+                for (int hf = 0; hf < HALVES; ++hf) {
+                  const int first = 16 * hf + 4 * kg;
+                  const int r0 = row0 + first;
+                  float res[4];
+                  act_fwd_w<4>(a.act, v[hf], res);
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) res[r] *= v[HALVES + hf][r];
+                  // Fragment order: H goes out the way the down projection's MFMAs take it in,
+                  // [N/8][16 MT token slots][8 elements], so that a token-operand fragment there is
+                  // 4 runs of 256 MT bytes (one contiguous KiB for MT = 1) instead of 16 row pieces
+                  // of 64 bytes.  All slots are written (slots past M repeat the last token), so
+                  // nothing uninitialised is multiplied.
+                  if (first < valid) {
+                    if (a.tiled)
+                      store_w<T, 4>((T*)a.out + ((size_t)(r0 >> 3) * (16 * MT) + tok) * 8 + (r0 & 7), res);
+                    else
+                      store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + r0, res);
+                  }
                 }
               } else {
 #pragma unroll
-                for (int m = 0; m < NMAT; ++m)
-                  if (4 * kg + 16 * m < valid) store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + r0 + 16 * m, v[m]);
+                for (int g = 0; g < NREG; ++g)
+                  if (16 * g + 4 * kg < valid)
+                    store_w<T, 4>((T*)a.out + (size_t)tok * a.ldo + row0 + 16 * g + 4 * kg, v[g]);
               }
             }
           }
+          if (PARITIES == 1) {
+            // one buffer: nobody writes the next block's partial sums before wavefront 0 has read these
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            __builtin_amdgcn_s_barrier();
+          }
 #pragma unroll
-          for (int m = 0; m < NMAT; ++m)
+          for (int g = 0; g < NREG; ++g)
 #pragma unroll
-            for (int t = 0; t < MT; ++t) acc[m][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < MT; ++t) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
           ++blk;
         }
       }
@@ -325,11 +369,13 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_stream_kernel(StreamArgs
   wait_vmem<0>();
 }
 
-template <typename T, bool GATED, int NMAT, int MT>
+template <typename T, bool GATED, int NMAT, int MT, int SEGB>
 static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) {
-  constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT, MT) * NMAT * DS_REGION + 2 * (DS_WAVES - 1) * NMAT * MT * 256 * 4;
+  constexpr int NREG = NMAT * (512 / SEGB);
+  constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT, MT, SEGB) * NMAT * DS_REGION +
+                      ds_part_buffers(NMAT, MT, SEGB) * (DS_WAVES - 1) * NREG * MT * 256 * 4;
   static_assert(LDS <= 160 * 1024, "a workgroup has 160 KiB of LDS");
-  auto kern = decode_stream_kernel<T, GATED, NMAT, MT>;
+  auto kern = decode_stream_kernel<T, GATED, NMAT, MT, SEGB>;
   static LdsAttrOnce lds_attr;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
   // one workgroup per CU, each with its share of the rows; fewer when that would be under 16 rows
@@ -358,15 +404,24 @@ hipError_t launch_decode_stream(const T* x, const T* wg, const T* wu, const T* w
   if (num_cu <= 0) num_cu = 256;
   const int tiled = ds_h_tiled(M);
   StreamArgs a1 = {x, {wg, wu}, {bg, bu}, h, M, N, K, K, N, act, tiled};
-  StreamArgs a2 = {h, {wd, wd + (size_t)16 * N}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY, tiled};
-  // 32-row blocks halve the L2 traffic for H; worth it when a CU's share of the rows exceeds 16
+  StreamArgs a2 = {h, {wd, wd}, {bd, bd}, y, M, K, N, N, K, ACT_IDENTITY, tiled};
+  // two runs of W_down rows per token-operand fetch halve the L2 traffic for H; worth it when a
+  // CU's share of the rows exceeds one run
   const bool wide = K > 16 * num_cu;
   if (M <= 16) {
-    if (hipError_t e = launch_stream<T, true, 2, 1>(a1, num_cu, s)) return e;
-    return wide ? launch_stream<T, false, 2, 1>(a2, num_cu, s) : launch_stream<T, false, 1, 1>(a2, num_cu, s);
+    if (hipError_t e = launch_stream<T, true, 2, 1, 512>(a1, num_cu, s)) return e;
+    return wide ? launch_stream<T, false, 2, 1, 512>(a2, num_cu, s) : launch_stream<T, false, 1, 1, 512>(a2, num_cu, s);
   }
-  if (hipError_t e = launch_stream<T, true, 2, 2>(a1, num_cu, s)) return e;
-  return wide ? launch_stream<T, false, 2, 2>(a2, num_cu, s) : launch_stream<T, false, 1, 2>(a2, num_cu, s);
+  // Two token tiles.  With 512-byte row segments the token operands cost as much L2 traffic as
+  // the weights cost HBM traffic, and the time grows by about 2 us per token at the 70B widths;
+  // 256-byte segments over twice the rows halve that but stream a few per cent slower from HBM.
+  // The two cross between M = 20 and M = 24 at every width measured.
+  if (M <= DS_WIDE_SEGMENT_MAX_M) {
+    if (hipError_t e = launch_stream<T, true, 2, 2, 512>(a1, num_cu, s)) return e;
+    return wide ? launch_stream<T, false, 2, 2, 512>(a2, num_cu, s) : launch_stream<T, false, 1, 2, 512>(a2, num_cu, s);
+  }
+  if (hipError_t e = launch_stream<T, true, 2, 2, 256>(a1, num_cu, s)) return e;
+  return wide ? launch_stream<T, false, 2, 2, 256>(a2, num_cu, s) : launch_stream<T, false, 1, 2, 256>(a2, num_cu, s);
 }
 
 template hipError_t launch_decode_stream<f16>(const f16*, const f16*, const f16*, const f16*,

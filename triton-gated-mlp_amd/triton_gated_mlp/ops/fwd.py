@@ -128,7 +128,7 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
 
 
 DECODE_MAX_M = 32
-DECODE_PREFERRED_MAX_M = 20
+DECODE_PREFERRED_MAX_M = 32
 
 
 def max_rows_32bit(K: int, N: int, dtype: torch.dtype) -> Optional[int]:
@@ -165,9 +165,8 @@ def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16,
     a block of W_gate/W_up rows and half a block of W_down rows; from there they beat or match the
     general path (GEMMs with split reductions) for every M <= 16 (measured on MI355X at the widths
     of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384 and 2048 x 8192).  With two token tiles
-    (16 < M <= 32) the token operands cost as much L2 traffic as the weights cost HBM traffic: the
-    kernels still win by 4 to 11 % at M = 17 and draw level between M = 24 and 32, so the module
-    takes them up to M = 20.
+    (16 < M <= 32) the token operands cost L2 traffic of the order of the weights' HBM traffic: the
+    kernels win by 4 to 11 % at M = 17 and by 0 to 5 % at M = 24 and 32.
     """
     return M <= DECODE_PREFERRED_MAX_M and decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu and K >= 8 * num_cu
 
