@@ -661,15 +661,18 @@ def test_decode_with_two_token_tiles(dtype):
                            torch.zeros(512, 1024, dtype=dtype, device=dev), None)
 
 
-@pytest.mark.parametrize("M,K,N", [(8, 1024, 4096), (64, 1024, 4096)])
-def test_inference_forward_under_hip_graph_replay(M, K, N):
-    """Serving loops replay a captured forward: the skinny-M streaming path (M = 8) and the general
-    path with split reductions (M = 64) are captured once and replayed with new inputs written into
-    the captured input buffer; every replay must equal the eager result for that input, with eager
-    work and synchronisations in between."""
+@pytest.mark.parametrize("M,K,N,streams", [(8, 2048, 4096, True), (24, 2048, 4096, True), (64, 1024, 4096, False)])
+def test_inference_forward_under_hip_graph_replay(M, K, N, streams):
+    """Serving loops replay a captured forward: the skinny-M streaming path (one and two token
+    tiles) and the general path with split reductions are captured once and replayed with new
+    inputs written into the captured input buffer; every replay must equal the eager result for
+    that input, with eager work and synchronisations in between."""
     from triton_gated_mlp import FusedGatedMLP
+    from triton_gated_mlp.ops import fwd as ops_fwd
 
     dev = _dev()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    assert ops_fwd.decode_preferred(M, K, N, torch.float16, cus) == streams
     mlp = FusedGatedMLP(K, N, bias=True).to(dev).to(torch.float16).eval()
     g = torch.Generator().manual_seed(41)
     inputs = [torch.randn(M, K, generator=g).half().to(dev) for _ in range(3)]
