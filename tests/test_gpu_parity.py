@@ -661,7 +661,7 @@ def test_decode_with_two_token_tiles(dtype):
                            torch.zeros(512, 1024, dtype=dtype, device=dev), None)
 
 
-@pytest.mark.parametrize("M,K,N,streams", [(8, 2048, 4096, True), (24, 2048, 4096, True), (64, 1024, 4096, False)])
+@pytest.mark.parametrize("M,K,N,streams", [(8, 2048, 4096, True), (24, 3584, 4096, True), (64, 1024, 4096, False)])
 def test_inference_forward_under_hip_graph_replay(M, K, N, streams):
     """Serving loops replay a captured forward: the skinny-M streaming path (one and two token
     tiles) and the general path with split reductions are captured once and replayed with new

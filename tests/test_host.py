@@ -258,6 +258,8 @@ def test_decode_preferred_needs_widths_that_fill_the_chip():
         assert all(decode_preferred(M, K, N) for M in (1, 8, 9, 16)), (K, N)
     assert decode_preferred(17, 8192, 28672) and decode_preferred(32, 4096, 14336)  # two token tiles
     assert not decode_preferred(33, 8192, 28672)  # beyond the skinny-M kernels
+    assert decode_preferred(16, 2560, 10240) and not decode_preferred(17, 2560, 10240)  # two tiles want wider models
+    assert decode_preferred(24, 3584, 18944)
     assert not decode_preferred(1, 4096 + 64, 14336)  # K must be a multiple of 256 for the streaming kernels
     assert not decode_preferred(1, 1024, 2048)  # fewer W_gate/W_up blocks than compute units
     assert not decode_preferred(1, 1024, 8192)  # a quarter of a W_down block per compute unit

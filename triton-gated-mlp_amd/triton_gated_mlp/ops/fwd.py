@@ -166,9 +166,13 @@ def decode_preferred(M: int, K: int, N: int, dtype: torch.dtype = torch.float16,
     general path (GEMMs with split reductions) for every M <= 16 (measured on MI355X at the widths
     of Llama-2-7B/13B, Llama-3-8B/70B, 6144 x 16384 and 2048 x 8192).  With two token tiles
     (16 < M <= 32) the token operands cost L2 traffic of the order of the weights' HBM traffic: the
-    kernels win by 4 to 11 % at M = 17 and by 0 to 5 % at M = 24 and 32.
+    kernels win by 4 to 17 % at M = 17 and by 0 to 10 % at M = 24 and 32 for hidden sizes from 3584
+    up; below that they tie or lose (2560 x 10240: -12 %), so the module asks for 14 rows of W_down
+    per compute unit there.
     """
-    return M <= DECODE_PREFERRED_MAX_M and decode_supported(M, K, N, dtype) and K % 256 == 0 and N >= 16 * num_cu and K >= 8 * num_cu
+    if M > DECODE_PREFERRED_MAX_M or not decode_supported(M, K, N, dtype) or K % 256 != 0 or N < 16 * num_cu:
+        return False
+    return K >= (8 if M <= 16 else 14) * num_cu
 
 
 def decode_fwd(
