@@ -1,30 +1,32 @@
 // Skinny-M (M <= 32) weight-streaming kernels, HBM-bound: every weight byte is fetched once, in
-// 512-byte row segments moved global -> LDS without passing through registers.
+// 512-byte (or 256-byte) row segments moved global -> LDS without passing through registers.
 //
 // One persistent workgroup of three wavefronts per CU.  The workgroup takes blocks of weight rows
 // that share one set of token operands: rows r..r+15 of W_gate and of W_up (GATED), or 32
-// consecutive rows of W_down (16 when a CU's share is no more than that); whole blocks go round-robin
-// over the workgroups, the rows that do not fill a last round are shared out evenly as one partly
-// empty block each.  Its wavefronts split the reduction range in
-// near-equal runs of 256-element chunks and combine their partial sums through LDS at the
-// end of each block (fixed order, so the result is deterministic).  Each wavefront runs a private
-// ring of 3 LDS slots; a slot holds one stage = 256 reduction elements of the 16 weight rows of
-// each matrix.  The matching token-row operands (x or H, L2-resident) are fetched straight into
-// registers, three stages ahead as well: one 16-token tile for M <= 16, two beyond (MT; the weight
-// fragment read from LDS then feeds two MFMAs).  Achieved HBM bandwidth follows the bytes in flight per
-// CU, and LDS capacity bounds those: wavefronts x 3 slots x slot size fill 144 of the 160 KiB.
-// The stream of stages runs on across block boundaries, so the ring never drains; loads past the
-// end re-fetch the last stage into a free slot, which keeps the in-flight count constant.
+// consecutive rows of W_down (16 when a CU's share is no more than that); twice as many rows with
+// 256-byte segments.  Whole blocks go round-robin over the workgroups, the rows that do not fill a
+// last round are shared out evenly as one partly empty block each.  Its wavefronts split the
+// reduction range in near-equal runs of chunks (256 or 128 elements) and combine their partial
+// sums through LDS at the end of each block (fixed order, so the result is deterministic).  Each
+// wavefront runs a private ring of 3 or 4 LDS slots; a slot holds one stage = one chunk of the
+// block's weight rows, 8 KiB per matrix.  The matching token-row operands (x or H, L2-resident)
+// are fetched straight into registers, as many stages ahead: one 16-token tile for M <= 16, two
+// beyond (MT; the weight fragment read from LDS then feeds two MFMAs).  Achieved HBM bandwidth
+// follows the bytes in flight per CU, and LDS capacity bounds those: wavefronts x 3 slots x 16 KiB
+// fill 144 of the 160 KiB.  The stream of stages runs on across block boundaries, so the ring
+// never drains; loads past the end re-fetch the last stage into a free slot, which keeps the
+// in-flight count constant.
 //
 //   GATED:   H[m, r] = act(x.W_gate[r] + b_gate[r]) * (x.W_up[r] + b_up[r])      (r over N)
 //   !GATED:  Y[m, r] = H.W_down[r] + b_down[r]                                   (r over K)
 //
-// LDS layout of a slot: 2 regions of 16 rows x 512 bytes; the 16-byte chunk c of row r is
-// stored at position c ^ r, so the 16 lanes that read one chunk index of 16 different rows for
-// v_mfma_f32_16x16x32 hit 16 different bank groups.
+// LDS layout of a slot: regions of 16 rows x SEGB bytes (SEGB = 512 or 256); the 16-byte chunk c
+// of row r is stored at position c ^ r, so the 16 lanes that read one chunk index of 16 different
+// rows for v_mfma_f32_16x16x32 hit 16 different bank groups.
 //
 // All vector-memory loads of the main loop are written as assembly and ordered by explicit
-// s_waitcnt vmcnt(N): the compiler does not see them, so it cannot serialise them either.
+// s_waitcnt vmcnt(N): the compiler does not see them, so it cannot serialise them either (the
+// build checks the generated assembly for uses of a load's destination ahead of its wait).
 #include "launch.hpp"
 #include "lds_dma.hpp"
 
