@@ -387,6 +387,55 @@ def test_forward_mask_output_equals_standalone_mask():
     _close("U", hs.up, o["U"])
 
 
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_gateup_as_whole_rounds_plus_remaining_columns(with_mask):
+    """A grid of large tiles that ends in a thinly filled round of workgroups is launched as two
+    column ranges (here 352 tiles on 256 compute units: 32 tile columns, then 12 on small tiles).
+    Biases, kept G and U, and the dropout mask must line up across the seam: the mask of an element
+    depends on its index in the whole tensor.  With and without the keep-mask output (the two
+    epilogue implementations)."""
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(6)
+    M, K, N, p = 2048, 64, 5632, 0.3
+    x = torch.randn(M, K, generator=g).half().to(dev)
+    Wg = (0.1 * torch.randn(N, K, generator=g)).half().to(dev)
+    Wu = (0.1 * torch.randn(N, K, generator=g)).half().to(dev)
+    bg = (0.1 * torch.randn(N, generator=g)).half().to(dev)
+    bu = (0.1 * torch.randn(N, generator=g)).half().to(dev)
+    hs = ops_fwd.gateup_fwd(x, Wg, bg, Wu, bu, p, seed=123, offset=2, save_activations=True, return_mask=with_mask)
+    ref = philox.keep_mask(M, N, p, 123, 2)
+    if with_mask:
+        assert np.array_equal(hs.mask.cpu().numpy(), ref)
+    f = lambda t: t.float().cpu()
+    o = oracle.hidden_forward(f(x), f(Wg), f(bg), f(Wu), f(bu), torch.from_numpy(ref), p)
+    _close("H", hs.hidden, o["H"])
+    _close("G", hs.gate, o["G"])
+    _close("U", hs.up, o["U"])
+    # dropped elements are exact zeros, kept ones are not (up to the odd underflow): the mask
+    # itself, read off H on both sides of the seam at column 4096
+    zero = (hs.hidden == 0).cpu().numpy()
+    assert (zero[:, :4096] == (ref[:, :4096] == 0)).mean() > 0.999
+    assert (zero[:, 4096:] == (ref[:, 4096:] == 0)).mean() > 0.999
+
+
+def test_linear_as_whole_rounds_plus_remaining_columns():
+    """The same two-launch form for the plain projection: 352 large tiles on 256 compute units,
+    bias included; also a shape with exactly one round, which must stay a single launch's result."""
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(8)
+    for M, R, C in [(2048, 64, 11264), (2048, 64, 8192)]:
+        a = torch.randn(M, R, generator=g).half().to(dev)
+        W = (0.1 * torch.randn(C, R, generator=g)).half().to(dev)
+        b = (0.1 * torch.randn(C, generator=g)).half().to(dev)
+        y = ops_fwd.linear_fwd(a, W, b)
+        ref = a.float().cpu() @ W.float().cpu().T + b.float().cpu()
+        _close(f"linear {M}x{R}->{C}", y, ref)
+
+
 def test_full_size_properties_cfg3_linearity_and_zero():
     """Size-independent checks at the headline shape: x = 0 gives Y = 0 (no bias), and the down
     projection is linear in H (Y(2H) = 2Y(H))."""

@@ -399,6 +399,9 @@ struct EpiGateUp {
     int ldc;
     int act;            // Act code
     DropoutParams drop;
+    size_t drop_e0;     // element index, in the whole [M, ldc] tensor, of what h points at: the
+                        // dropout counter of an element is its index in the whole tensor, also
+                        // when a launch covers a range of columns only
   };
   // ACT: activation fixed at compile time, or ACT_RUNTIME to read a.act.  A kernel whose epilogue
   // is unrolled many times instantiates both and branches once, so that the usual SiLU path stays
@@ -416,7 +419,7 @@ struct EpiGateUp {
     for (int r = 0; r < W; ++r) h[r] *= u[r];
     if (a.drop.enabled) {
       bool keep[W];
-      keep_w<W>(a.drop, e, keep);
+      keep_w<W>(a.drop, e + a.drop_e0, keep);
 #pragma unroll
       for (int r = 0; r < W; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
       if (a.mask_out) {
@@ -487,7 +490,7 @@ struct EpiGateUpPacked : EpiGateUp<T> {
     for (int r = 0; r < 4; ++r) h[r] *= u[r];
     if (a.drop.enabled) {
       bool keep[4];
-      keep_w<4>(a.drop, (size_t)m * a.ldc + n, keep);
+      keep_w<4>(a.drop, (size_t)m * a.ldc + n + a.drop_e0, keep);
 #pragma unroll
       for (int r = 0; r < 4; ++r) h[r] = keep[r] ? h[r] * a.drop.scale : 0.f;
     }
