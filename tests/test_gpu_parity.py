@@ -436,6 +436,38 @@ def test_linear_as_whole_rounds_plus_remaining_columns():
         _close(f"linear {M}x{R}->{C}", y, ref)
 
 
+def test_backward_gemms_as_whole_rounds_plus_remaining_rows():
+    """dH (with the gating-backward epilogue and dropout) and dX with 352 large tiles on 256 compute
+    units: launched as 11 tile rows that make a whole round plus the remaining 5 as a problem of
+    their own.  G, U, dG, dU and the dropout counters must line up across the seam at row 2816."""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(9)
+    M, K, N, p = 4096, 64, 5632, 0.25
+    dy = torch.randn(M, K, generator=g).half().to(dev)
+    Wd = (0.1 * torch.randn(K, N, generator=g)).half().to(dev)
+    G = torch.randn(M, N, generator=g).half().to(dev)
+    U = torch.randn(M, N, generator=g).half().to(dev)
+    dg, du = ops_bwd.dh_bwd(dy, Wd, G, U, p, 321, 4)
+    keep = torch.from_numpy(philox.keep_mask(M, N, p, 321, 4))
+    f = lambda t: t.float().cpu()
+    ref = oracle.hidden_backward(f(dy) @ f(Wd), f(G), f(U), keep, p)
+    _close("dG", dg, ref["dG"])
+    _close("dU", du, ref["dU"])
+    zero = (du == 0).cpu().numpy()
+    for rows in (slice(0, 2816), slice(2816, M)):
+        assert (zero[rows] == (keep[rows].numpy() == 0)).mean() > 0.999
+
+    M, K, N = 4096, 5632, 64
+    dG = torch.randn(M, N, generator=g).half().to(dev)
+    dU = torch.randn(M, N, generator=g).half().to(dev)
+    Wg = (0.1 * torch.randn(N, K, generator=g)).half().to(dev)
+    Wu = (0.1 * torch.randn(N, K, generator=g)).half().to(dev)
+    dx = ops_bwd.dx_bwd(dG, dU, Wg, Wu)
+    _close("dX", dx, f(dG) @ f(Wg) + f(dU) @ f(Wu))
+
+
 def test_full_size_properties_cfg3_linearity_and_zero():
     """Size-independent checks at the headline shape: x = 0 gives Y = 0 (no bias), and the down
     projection is linear in H (Y(2H) = 2Y(H))."""

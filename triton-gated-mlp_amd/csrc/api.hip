@@ -156,6 +156,19 @@ int pick_splits(int dtype, int64_t rows, int64_t cols, int64_t red, int64_t red_
   return (int)((red_tiles + per - 1) / per);
 }
 
+// For a rows x cols output on 256 x 256 tiles whose grid ends in a thinly filled round of
+// workgroups (at most half full): the number of tile ROWS that make whole rounds, or 0.  The
+// backward GEMMs read their weight operand reduction-strided, so they are cut along the rows of
+// the output (token rows: every other operand is row-major in them) where the forward GEMMs are cut
+// along the columns.
+int64_t whole_round_tile_rows(int dtype, int64_t rows, int64_t cols, int64_t red) {
+  if (dtype == GMLP_F32 || pick_tile(dtype, rows, cols, red, 256) != gmlp::TILE_LARGE) return 0;
+  const int64_t tiles_m = (rows + 255) / 256, tiles_n = (cols + 255) / 256, cus = num_cu();
+  const int64_t rounds = tiles_m * tiles_n / cus, tail = tiles_m * tiles_n % cus;
+  const int64_t whole = rounds * cus / tiles_n;
+  return rounds >= 1 && tail > 0 && 2 * tail <= cus && whole >= 1 && whole < tiles_m ? whole : 0;
+}
+
 size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols, int accumulator_sets = 1) {
   return splits > 1 ? (size_t)splits * accumulator_sets * rows * cols * sizeof(float) : 0;
 }
@@ -311,16 +324,25 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   GMLP_REQUIRE_ALIGNED(u); GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du);
 
   // dH[M,N] = dY[M,K] · W_down[K,N]: reduction over K; B is reduction-strided ([K,N] row-major).
-  GemmArgs ga = {};
-  ga.A[0] = dy; ga.A[1] = dy; ga.B[0] = w_down; ga.B[1] = w_down;
-  ga.M = (int)M; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
-  ga.nseg = 1; ga.group_m = pick_group(M, N);
-  int tc = pick_tile(dtype, M, N, K, 256);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e = by_dtype(dtype, [&](auto tag) {
+  hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
-    typename EpiDh<T>::Args ea = {(const T*)g, (const T*)u, (T*)dg, (T*)du, (int)N, act, d};
-    return launch_dh<T>(tc, ga, ea, s);
+    // The GEMM over output rows [row0, row0 + rows): every per-row pointer moves along.
+    auto run = [&](int64_t row0, int64_t rows, int force_class) -> hipError_t {
+      GemmArgs ga = {};
+      ga.A[0] = (const T*)dy + row0 * K; ga.A[1] = ga.A[0]; ga.B[0] = w_down; ga.B[1] = w_down;
+      ga.M = (int)rows; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
+      ga.nseg = 1; ga.group_m = pick_group(rows, N);
+      const size_t e0 = (size_t)row0 * N;
+      typename EpiDh<T>::Args ea = {(const T*)g + e0, (const T*)u + e0, (T*)dg + e0, (T*)du + e0, (int)N, act, d, e0};
+      return launch_dh<T>(force_class >= 0 ? force_class : pick_tile(dtype, rows, N, K, 256), ga, ea, s);
+    };
+    int64_t whole = whole_round_tile_rows(dtype, M, N, K);
+    if (whole > 0) {
+      if (hipError_t err = run(0, whole * 256, TILE_LARGE)) return err;
+      return run(whole * 256, M - whole * 256, -1);
+    }
+    return run(0, M, -1);
   });
   return hip_result(__func__, e);
 }
@@ -361,27 +383,33 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   GMLP_REQUIRE_ALIGNED(w_up); GMLP_REQUIRE_ALIGNED(dx); GMLP_REQUIRE_ALIGNED(workspace);
 
   // dX[M,K] = dG[M,N]·W_gate[N,K] + dU[M,N]·W_up[N,K]: two reduction segments of length N.
-  GemmArgs ga = {};
-  ga.A[0] = dg; ga.A[1] = du; ga.B[0] = w_gate; ga.B[1] = w_up;
-  ga.M = (int)M; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
-  ga.nseg = 2; ga.group_m = pick_group(M, K); ga.rotate = M <= 512;
-  int tc = pick_tile(dtype, M, K, N, 256);
-  const int splits = pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64));
-  const bool split = splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, M, K);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
-    if constexpr (!std::is_same<T, float>::value) {
-      if (split) {
-        ga.splits = splits;
-        typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)M * K, 0, (int)K};
-        if (hipError_t err = launch_dx_split<T>(ga, pa, s)) return err;
-        typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};
-        return launch_splitk_reduce<T, EpiStore<T>>((const float*)workspace, splits, (size_t)M * K, 0, ea, M, K, s);
+    // The GEMM over output rows [row0, row0 + rows).
+    auto run = [&](int64_t row0, int64_t rows, bool may_split, int force_class) -> hipError_t {
+      GemmArgs ga = {};
+      ga.A[0] = (const T*)dg + row0 * N; ga.A[1] = (const T*)du + row0 * N; ga.B[0] = w_gate; ga.B[1] = w_up;
+      ga.M = (int)rows; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
+      ga.nseg = 2; ga.group_m = pick_group(rows, K); ga.rotate = rows <= 512;
+      typename EpiStore<T>::Args ea = {(T*)dx + row0 * K, nullptr, (int)K};
+      if constexpr (!std::is_same<T, float>::value) {
+        const int splits = may_split ? pick_splits(dtype, rows, K, N, 2 * ((N + 63) / 64)) : 1;
+        if (splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(splits, rows, K)) {
+          ga.splits = splits;
+          typename EpiPartial<T>::Args pa = {(float*)workspace, (size_t)rows * K, 0, (int)K};
+          if (hipError_t err = launch_dx_split<T>(ga, pa, s)) return err;
+          return launch_splitk_reduce<T, EpiStore<T>>((const float*)workspace, splits, (size_t)rows * K, 0, ea, rows, K, s);
+        }
       }
+      return launch_dx<T>(force_class >= 0 ? force_class : pick_tile(dtype, rows, K, N, 256), ga, ea, s);
+    };
+    int64_t whole = whole_round_tile_rows(dtype, M, K, N);
+    if (whole > 0) {
+      if (hipError_t err = run(0, whole * 256, false, TILE_LARGE)) return err;
+      return run(whole * 256, M - whole * 256, false, -1);
     }
-    typename EpiStore<T>::Args ea = {(T*)dx, nullptr, (int)K};
-    return launch_dx<T>(tc, ga, ea, s);
+    return run(0, M, true, -1);
   });
   return hip_result(__func__, e);
 }

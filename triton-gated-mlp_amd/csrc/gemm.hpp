@@ -507,11 +507,12 @@ struct EpiGateUpPacked : EpiGateUp<T> {
 template <typename T, int W, int ACT = ACT_RUNTIME>
 __device__ __forceinline__ void gating_bwd_core(int act, const DropoutParams& drop, size_t e, float* dh,
                                                 typename PackW<T, W>::type gp,
-                                                typename PackW<T, W>::type up, T* dg, T* du) {
+                                                typename PackW<T, W>::type up, T* dg, T* du,
+                                                size_t drop_e0 = 0) {
   float dgv[W], duv[W];
   if (drop.enabled) {
     bool keep[W];
-    keep_w<W>(drop, e, keep);
+    keep_w<W>(drop, e + drop_e0, keep);  // drop_e0: see EpiGateUp::Args
 #pragma unroll
     for (int r = 0; r < W; ++r) dh[r] = keep[r] ? dh[r] * drop.scale : 0.f;
   }
@@ -529,9 +530,10 @@ __device__ __forceinline__ void gating_bwd_core(int act, const DropoutParams& dr
 }
 template <typename T, int W>
 __device__ __forceinline__ void gating_bwd_w(int act, const DropoutParams& drop, size_t e,
-                                             float* dh, const T* g, const T* u, T* dg, T* du) {
+                                             float* dh, const T* g, const T* u, T* dg, T* du,
+                                             size_t drop_e0 = 0) {
   typedef typename PackW<T, W>::type pack;
-  gating_bwd_core<T, W>(act, drop, e, dh, *(const pack*)(g + e), *(const pack*)(u + e), dg, du);
+  gating_bwd_core<T, W>(act, drop, e, dh, *(const pack*)(g + e), *(const pack*)(u + e), dg, du, drop_e0);
 }
 
 template <typename T>
@@ -544,10 +546,11 @@ struct EpiDh {
     int ldc;
     int act;  // Act code
     DropoutParams drop;
+    size_t drop_e0;  // see EpiGateUp::Args
   };
   template <int W>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*) {
-    gating_bwd_w<T, W>(a.act, a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du);
+    gating_bwd_w<T, W>(a.act, a.drop, (size_t)m * a.ldc + n, dh, a.g, a.u, a.dg, a.du, a.drop_e0);
   }
   // G and U come from HBM and every workgroup of a round reaches its epilogue at about the same
   // time; a kernel that can, fetches them this many W-wide items ahead of their use.
@@ -569,7 +572,7 @@ struct EpiDh {
   template <int W, int ACT>
   static __device__ __forceinline__ void apply(const Args& a, int m, int n, float* dh, float*,
                                                const Prefetch<W>& p) {
-    gating_bwd_core<T, W, ACT>(a.act, a.drop, (size_t)m * a.ldc + n, dh, p.g, p.u, a.dg, a.du);
+    gating_bwd_core<T, W, ACT>(a.act, a.drop, (size_t)m * a.ldc + n, dh, p.g, p.u, a.dg, a.du, a.drop_e0);
   }
 };
 
