@@ -468,6 +468,27 @@ def test_backward_gemms_as_whole_rounds_plus_remaining_rows():
     _close("dX", dx, f(dG) @ f(Wg) + f(dU) @ f(Wu))
 
 
+@pytest.mark.parametrize("band", ["columns", "rows"])
+def test_grouped_weight_gradients_with_a_band_of_the_last_problem_on_its_own(band):
+    """528 large tiles on 256 compute units: the last problem of the group gives up a band of 16
+    tiles (two tile columns, or two tile rows when it is the tall one), which runs as a launch of
+    its own through a moved pointer and a trimmed buffer size.  A reduction length that is not a
+    multiple of 64 makes the trimmed size matter: reduction rows past the end must read as zero."""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(10)
+    Mred = 200
+    shapes = [(5632, 2048), (5632, 2048), (2048, 5632)] if band == "columns" else [(2048, 5632), (2048, 5632), (5632, 2048)]
+    pairs = []
+    for R, C in shapes:
+        pairs.append((torch.randn(Mred, R, generator=g).half().to(dev), torch.randn(Mred, C, generator=g).half().to(dev)))
+    outs = ops_bwd.dw_bwd_grouped(pairs)
+    for (lhs, rhs), out in zip(pairs, outs):
+        ref = lhs.float().cpu().T @ rhs.float().cpu()
+        _close(f"dW {tuple(out.shape)}", out, ref)
+
+
 def test_full_size_properties_cfg3_linearity_and_zero():
     """Size-independent checks at the headline shape: x = 0 gives Y = 0 (no bias), and the down
     projection is linear in H (Y(2H) = 2Y(H))."""

@@ -476,6 +476,26 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
     ga.M = (int)R[i]; ga.N = (int)C[i]; ga.K = (int)Mred; ga.lda = (int)R[i]; ga.ldb = (int)C[i];
     ga.nseg = 1; ga.group_m = pick_group(R[i], C[i]);
   };
+  // A grid of large tiles that ends in a thinly filled round: the last problem gives up a band of
+  // its output (whole tile rows or tile columns, whichever comes closer to the tiles of that last
+  // round), which runs as a launch of its own on the tile class that suits it; the rest then makes
+  // whole rounds.  Both operands are reduction-strided, so the band is a range of columns of one
+  // of them: the pointer moves along the rows and the buffer size is trimmed to match.
+  int64_t band_rows = 0, band_cols = 0;  // size of the band, in output rows or columns (one is 0)
+  const int last = count - 1;
+  if (group_class == TILE_LARGE) {
+    const int64_t cus = num_cu(), rounds = tiles256 / cus, tail = tiles256 % cus;
+    const int64_t tr = (R[last] + 255) / 256, tc = (C[last] + 255) / 256;
+    // (worth it for a few rounds only: measured -7 % at 2 rounds, -1 % and less from 8 rounds on)
+    if (rounds >= 1 && rounds <= 4 && tail > 0 && 2 * tail <= cus) {
+      const int64_t by_rows = (tail + tc - 1) / tc, by_cols = (tail + tr - 1) / tr;  // tile rows / columns
+      const bool rows_fit = by_rows < tr, cols_fit = by_cols < tc;
+      if (cols_fit && (!rows_fit || by_cols * tr <= by_rows * tc)) band_cols = C[last] - (tc - by_cols) * 256;
+      else if (rows_fit) band_rows = R[last] - (tr - by_rows) * 256;
+      const int64_t br = band_rows ? band_rows : R[last], bc = band_cols ? band_cols : C[last];
+      if ((band_rows || band_cols) && pick_tile(dtype, br, bc, Mred, 256, true) == TILE_MEDIUM) band_rows = band_cols = 0;
+    }
+  }
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
     if constexpr (std::is_same<T, float>::value) {
@@ -487,7 +507,22 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
         fill(grp.ga[i], i);
         grp.ea[i] = typename EpiStore<T>::Args{(T*)dw[i], nullptr, (int)C[i]};
       }
-      return launch_dw_group<T>(group_class, grp, s);
+      grp.ga[last].M -= (int)band_rows;
+      grp.ga[last].N -= (int)band_cols;
+      if (hipError_t err = launch_dw_group<T>(group_class, grp, s)) return err;
+      if (band_rows == 0 && band_cols == 0) return hipSuccess;
+      GemmArgs ga;
+      fill(ga, last);
+      const int64_t r0 = band_rows ? R[last] - band_rows : 0, c0 = band_cols ? C[last] - band_cols : 0;
+      ga.A[0] = ga.A[1] = (const T*)lhs[last] + r0;
+      ga.B[0] = ga.B[1] = (const T*)rhs[last] + c0;
+      ga.a_trim = (int)(r0 * sizeof(T));
+      ga.b_trim = (int)(c0 * sizeof(T));
+      ga.M = (int)(R[last] - r0);
+      ga.N = (int)(C[last] - c0);
+      ga.group_m = pick_group(ga.M, ga.N);
+      typename EpiStore<T>::Args ea = {(T*)dw[last] + r0 * C[last] + c0, nullptr, (int)C[last]};
+      return launch_dw<T>(pick_tile(dtype, ga.M, ga.N, Mred, 256, true), ga, ea, s);
     }
   });
   return hip_result(__func__, e);

@@ -29,6 +29,10 @@ struct GemmArgs {
   int splits;        // pipelined kernel with a split-reduction epilogue only: number of workgroups
                      // that share one output tile, each reducing a contiguous range of 64-wide
                      // reduction tiles into a partial result of its own (0 or 1: no split)
+  int a_trim, b_trim;  // pipelined kernel: bytes to take off the size of a reduction-strided operand
+                     // whose pointer has been moved along its rows to address a range of output
+                     // rows / columns (the operand then ends that many bytes earlier than its row
+                     // count times its pitch says)
   int rotate;        // pipelined kernel: the workgroups of tile column c start their reduction
                      // range at tile c mod length and wrap around.  For short batches, which are
                      // bound by streaming the B operand (the weights): the workgroups would

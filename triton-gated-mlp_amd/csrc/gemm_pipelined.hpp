@@ -164,8 +164,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const uint32_t a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
   const uint32_t b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem;
-  const uint32_t a_bytes = (uint32_t)(A_KS ? ga.K : ga.M) * ga.lda * 2 + DMA_BIAS;
-  const uint32_t b_bytes = (uint32_t)(B_KS ? ga.K : ga.N) * ga.ldb * 2 + DMA_BIAS;
+  const uint32_t a_bytes = (uint32_t)(A_KS ? ga.K : ga.M) * ga.lda * 2 + DMA_BIAS - (uint32_t)ga.a_trim;
+  const uint32_t b_bytes = (uint32_t)(B_KS ? ga.K : ga.N) * ga.ldb * 2 + DMA_BIAS - (uint32_t)ga.b_trim;
   const buffer_rsrc ra[2] = {make_rsrc((const char*)ga.A[0] - DMA_BIAS, a_bytes),
                              make_rsrc((const char*)ga.A[1] - DMA_BIAS, a_bytes)};
   const buffer_rsrc rb[2] = {make_rsrc((const char*)ga.B[0] - DMA_BIAS, b_bytes),
