@@ -380,8 +380,9 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
   auto kern = decode_stream_kernel<T, GATED, NMAT, MT, SEGB>;
   static LdsAttrOnce lds_attr;
   if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
-  // one workgroup per CU, each with its share of the rows; fewer when that would be under 16 rows
-  int grid = a.R / 16 < num_cu ? a.R / 16 : num_cu;
+  // one workgroup per CU, each with its share of the rows (a partly empty block when that is less
+  // than a block); fewer workgroups when a share would be under 8 rows
+  int grid = a.R / 8 < num_cu ? a.R / 8 : num_cu;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(DS_WAVES * 64), LDS, s, a);
   return hipGetLastError();
 }
