@@ -214,7 +214,9 @@ class FusedGatedMLP(_GatedMLPBase):
     Dropout is active in training mode only.  The keep mask comes from a counter-based generator:
     set `dropout_seed` (int) for a fixed mask stream, otherwise each forward draws a seed from
     torch's default CPU generator (so `torch.manual_seed` makes runs repeatable).  The seed and
-    offset of the last training forward are kept in `last_dropout_state`.
+    offset of the last training forward are kept in `last_dropout_state`; a batch that ran as
+    several row chunks (see `_forward_2d`) drew one mask per chunk, and `last_dropout_states` lists
+    them all as (first row, rows, seed, offset), the mask of a chunk being that of a [rows, N] tensor.
 
     Under `torch.autocast("cuda")` the module casts its input and parameters to the autocast dtype
     for the kernels (fp32 master weights keep fp32 gradients), as nn.Linear does.
@@ -229,6 +231,7 @@ class FusedGatedMLP(_GatedMLPBase):
         self.recompute_activations = False
         self._dropout_calls = 0
         self.last_dropout_state = (0, 0)
+        self.last_dropout_states = []
 
     def _next_dropout_state(self):
         if self.dropout_seed is None:
@@ -244,6 +247,7 @@ class FusedGatedMLP(_GatedMLPBase):
         x2 = x.reshape(-1, x.shape[-1])
         p = float(self.dropout.p) if self.training else 0.0
         gate, up, down = self.gate_proj, self.up_proj, self.down_proj
+        self.last_dropout_states = []
         if x2.is_cuda and torch.is_autocast_enabled("cuda"):
             # Mixed precision as nn.Linear does it under torch.autocast: activations and (master)
             # weights are cast to the autocast dtype for the kernels; autograd casts the gradients back.
@@ -260,18 +264,18 @@ class FusedGatedMLP(_GatedMLPBase):
             cast(x2), cast(g.weight), cast(g.bias), cast(u.weight), cast(u.bias), cast(d.weight), cast(d.bias), p
         )
 
-    def _forward_2d(self, x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p: float) -> Tensor:
+    def _forward_2d(self, x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p: float, row0: int = 0) -> Tensor:
         M, K = x2.shape
         limit = _fwd.max_rows_32bit(K, self.intermediate_size, x2.dtype) if x2.is_cuda else None
         if limit is not None and M > limit:
             # Token rows are independent: a batch too tall for the pipelined kernels' 32-bit operand
             # offsets runs as near-equal row chunks (autograd sums the chunks' weight gradients; with
-            # dropout every chunk draws its own mask and `last_dropout_state` is the last chunk's).
+            # dropout every chunk draws its own mask, recorded in `last_dropout_states`).
             chunks = -(-M // limit)
             rows = -(-M // (chunks * 256)) * 256
             return torch.cat(
                 [
-                    self._forward_2d(x2[i : i + rows], W_gate, b_gate, W_up, b_up, W_down, b_down, p)
+                    self._forward_2d(x2[i : i + rows], W_gate, b_gate, W_up, b_up, W_down, b_down, p, row0 + i)
                     for i in range(0, M, rows)
                 ]
             )
@@ -286,6 +290,8 @@ class FusedGatedMLP(_GatedMLPBase):
             hs = _fwd.gateup_fwd(x2, W_gate, b_gate, W_up, b_up, 0.0, 0, 0, save_activations=False, act_fn=self.act_fn)
             return _fwd.linear_fwd(hs.hidden, W_down, b_down)
         seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
+        if p > 0.0:
+            self.last_dropout_states.append((row0, M, seed, offset))
         return FusedGatedMLPFullFunction.apply(
             x2, W_gate, b_gate, W_up, b_up, W_down, b_down, p, seed, offset, self.recompute_activations, self.act_fn
         )
