@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 6
+#define GMLP_ABI_VERSION 7
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -71,6 +71,17 @@ enum gmlp_op {
 
 int gmlp_abi_version(void);
 const char* gmlp_last_error(void);
+
+/*
+ * Optional set-up for the current HIP device: makes every one-time runtime call the entry points
+ * would otherwise make at their first launch on that device (raising the dynamic-LDS limit of each
+ * kernel, reading the compute-unit count).  Call it once per device before capturing a stream into a HIP graph: those
+ * calls are not allowed during capture, and an entry point that still needs one while its stream
+ * is capturing returns GMLP_EHIP (hipErrorStreamCaptureUnsupported) instead of making it.
+ * No counterpart in the reference (Triton compiles and configures its kernels at first launch,
+ * src/triton_gated_mlp/ops/fwd.py:257-276).
+ */
+int gmlp_init(void);
 
 /*
  * Workspace bytes the caller must provide for `op` at the given problem size (0 if none), with
@@ -180,7 +191,8 @@ int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void*
  * for M <= 32, streaming each weight matrix from HBM exactly once.  h_scratch holds 16*N elements
  * of dtype for M <= 16 and 32*N beyond: the intermediate H for 16 or 32 token slots, in an order of
  * the library's choosing;
- * workspace: gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, M, K, N, dtype) bytes.  No dropout (inference).
+ * workspace: unused by the current kernels (gmlp_workspace_bytes(GMLP_OP_DECODE_FWD, ...) is 0): pass
+ * NULL.  The argument is kept so that the signature does not change.  No dropout (inference).
  * Same math as EagerGatedMLP.forward in eval mode (src/triton_gated_mlp/gated_mlp.py:92-98).
  * Requires K % 32 == 0 and N % 256 == 0 (the LDS-ring streaming kernels run when K % 256 == 0 too,
  * K >= 768, N >= 768 and K*N < 2^30; 16 < M <= 32 is accepted only then).

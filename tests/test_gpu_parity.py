@@ -881,6 +881,22 @@ def test_inference_forward_under_hip_graph_replay(M, K, N, streams):
             assert torch.equal(y, eager[rep]), f"replay with input {rep} differs from the eager forward"
 
 
+def test_training_step_under_stream_capture_is_refused(monkeypatch):
+    """A forward that records an autograd graph while its stream is being captured raises a
+    RuntimeError (no kernel is enqueued, nothing is captured); the capture state is simulated on
+    the host, no stream is actually captured here."""
+    from triton_gated_mlp import FusedGatedMLP
+
+    dev = _dev()
+    mlp = FusedGatedMLP(256, 512, bias=False).to(dev).half()
+    x = torch.randn(64, 256, device=dev, dtype=torch.float16, requires_grad=True)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="autograd graph"):
+        mlp(x)
+    with torch.no_grad():
+        assert mlp(x).shape == (64, 256)  # inference is not affected
+
+
 @pytest.mark.skip(
     reason="capturing the step with torch.cuda.graph ended in a host-side segmentation fault inside "
     "capture_end (hipStreamEndCapture) on this image; cause not established, so the case stays off the GPU"

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"libgmlp.so does not export {name}"
     assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
-    assert lib.gmlp_abi_version() == 6
+    assert lib.gmlp_abi_version() == 7
 
 
 def _buf(nbytes=4096):

@@ -3,9 +3,12 @@
 // so the error paths can be exercised on a machine without a GPU.
 #include "gmlp.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
+#include <vector>
 
 #include "launch.hpp"
 
@@ -92,15 +95,23 @@ int pick_group(int64_t rows, int64_t cols, int sets = 1) { return sets * cols < 
 
 // Compute units of the current device.
 int num_cu() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
+}
+
+// Accelerator dies (XCDs, each with an L2 of its own) behind the current device: the hardware
+// deals consecutive workgroup ids round-robin to them.  A gfx950 XCD has 32 active compute units,
+// so a whole MI355X shows 8 and a partition of it 4, 2 or 1.
+int num_xcd() {
+  int n = num_cu() / 32;
+  return n < 1 ? 1 : n > 8 ? 8 : n;
 }
 
 // LARGE or MEDIUM_FULL for a grid of `large_tiles` large or `medium_tiles` small tiles, by
@@ -173,12 +184,46 @@ size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols, int accumul
   return splits > 1 ? (size_t)splits * accumulator_sets * rows * cols * sizeof(float) : 0;
 }
 
+std::mutex& lds_registry_mutex() {
+  static std::mutex m;
+  return m;
+}
+std::vector<gmlp::LdsKernel*>& lds_registry() {
+  static std::vector<gmlp::LdsKernel*> v;
+  return v;
+}
+
 }  // namespace
+
+namespace gmlp {
+
+LdsKernel::LdsKernel(const void* k, int b) : kernel(k), bytes(b), done{} {
+  std::lock_guard<std::mutex> lock(lds_registry_mutex());
+  lds_registry().push_back(this);
+}
+
+hipError_t prepare_lds_kernels() {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  std::lock_guard<std::mutex> lock(lds_registry_mutex());
+  for (LdsKernel* k : lds_registry()) {
+    if (hipError_t e = hipFuncSetAttribute(k->kernel, hipFuncAttributeMaxDynamicSharedMemorySize, k->bytes)) return e;
+    if (dev >= 0 && dev < 64) k->done[dev].store(1, std::memory_order_release);
+  }
+  return hipSuccess;
+}
+
+}  // namespace gmlp
 
 extern "C" {
 
 int gmlp_abi_version(void) { return GMLP_ABI_VERSION; }
 const char* gmlp_last_error(void) { return g_err; }
+
+int gmlp_init(void) {
+  (void)num_cu();
+  return hip_result(__func__, gmlp::prepare_lds_kernels());
+}
 
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {
   if (M < 1 || N < 1) return 0;
@@ -220,6 +265,7 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
     // row pitch of the outputs stays N.
     auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class) -> hipError_t {
       GemmArgs ga = {};
+      ga.nxcd = num_xcd();
       ga.A[0] = x; ga.A[1] = x;
       ga.B[0] = (const T*)w_gate + col0 * K; ga.B[1] = (const T*)w_up + col0 * K;
       ga.M = (int)M; ga.N = (int)cols; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
@@ -275,6 +321,7 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
     // The GEMM over output columns [col0, col0 + cols); the row pitch of `out` stays C.
     auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class) -> hipError_t {
       GemmArgs ga = {};
+      ga.nxcd = num_xcd();
       ga.A[0] = a; ga.A[1] = a;
       ga.B[0] = (const T*)w + col0 * R; ga.B[1] = ga.B[0];
       ga.M = (int)M; ga.N = (int)cols; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
@@ -330,6 +377,7 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
     // The GEMM over output rows [row0, row0 + rows): every per-row pointer moves along.
     auto run = [&](int64_t row0, int64_t rows, int force_class) -> hipError_t {
       GemmArgs ga = {};
+      ga.nxcd = num_xcd();
       ga.A[0] = (const T*)dy + row0 * K; ga.A[1] = ga.A[0]; ga.B[0] = w_down; ga.B[1] = w_down;
       ga.M = (int)rows; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
       ga.nseg = 1; ga.group_m = pick_group(rows, N);
@@ -389,6 +437,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
     // The GEMM over output rows [row0, row0 + rows).
     auto run = [&](int64_t row0, int64_t rows, bool may_split, int force_class) -> hipError_t {
       GemmArgs ga = {};
+      ga.nxcd = num_xcd();
       ga.A[0] = (const T*)dg + row0 * N; ga.A[1] = (const T*)du + row0 * N; ga.B[0] = w_gate; ga.B[1] = w_up;
       ga.M = (int)rows; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
       ga.nseg = 2; ga.group_m = pick_group(rows, K); ga.rotate = rows <= 512;
@@ -426,6 +475,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
 
   // dW[R,C] = lhs[Mred,R]ᵀ · rhs[Mred,C]: both operands reduction-strided.
   GemmArgs ga = {};
+      ga.nxcd = num_xcd();
   ga.A[0] = lhs; ga.A[1] = lhs; ga.B[0] = rhs; ga.B[1] = rhs;
   ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
   ga.nseg = 1; ga.group_m = pick_group(R, C);
@@ -472,6 +522,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
   hipStream_t s = (hipStream_t)stream;
   auto fill = [&](GemmArgs& ga, int i) {
     ga = GemmArgs{};
+    ga.nxcd = num_xcd();
     ga.A[0] = lhs[i]; ga.A[1] = lhs[i]; ga.B[0] = rhs[i]; ga.B[1] = rhs[i];
     ga.M = (int)R[i]; ga.N = (int)C[i]; ga.K = (int)Mred; ga.lda = (int)R[i]; ga.ldb = (int)C[i];
     ga.nseg = 1; ga.group_m = pick_group(R[i], C[i]);

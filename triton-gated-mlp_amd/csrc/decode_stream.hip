@@ -377,9 +377,8 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
   constexpr int LDS = DS_WAVES * ds_ring_depth(NMAT, MT, SEGB) * NMAT * DS_REGION +
                       ds_part_buffers(NMAT, MT, SEGB) * (DS_WAVES - 1) * NREG * MT * 256 * 4;
   static_assert(LDS <= 160 * 1024, "a workgroup has 160 KiB of LDS");
-  auto kern = decode_stream_kernel<T, GATED, NMAT, MT, SEGB>;
-  static LdsAttrOnce lds_attr;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, LDS, lds_attr)) return e;
+  constexpr auto kern = decode_stream_kernel<T, GATED, NMAT, MT, SEGB>;
+  if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, LDS>, s)) return e;
   // one workgroup per CU, each with its share of the rows (a partly empty block when that is less
   // than a block); fewer workgroups when a share would be under 8 rows
   int grid = a.R / 8 < num_cu ? a.R / 8 : num_cu;

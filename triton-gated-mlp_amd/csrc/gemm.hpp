@@ -40,16 +40,18 @@ struct GemmArgs {
                      // for the usual power-of-two row pitches crowds onto a few memory channels.
                      // Workgroups that share B rows keep the same order, so they still share them
                      // in L2.
+  int nxcd;          // accelerator dies of the device (each with its own L2) the hardware deals
+                     // workgroup ids to, round-robin (0 is read as 1: no remapping)
 };
 
 // Workgroup id -> output tile.  The hardware deals consecutive workgroup ids round-robin to the
-// 8 XCDs (each with its own L2); xcd_contiguous undoes that so each XCD walks a contiguous run of
-// indices, and tile_of walks tiles in groups of `group_m` tile-rows (column-major inside a group)
-// for operand reuse in L2.
-__device__ __forceinline__ int xcd_contiguous(int pid, int nwg) {
-  const int NXCD = 8;
-  int xcd = pid % NXCD, loc = pid / NXCD;
-  int per = nwg / NXCD, rem = nwg % NXCD;
+// device's XCDs (each with its own L2; 8 on a whole MI355X); xcd_contiguous undoes that so each XCD
+// walks a contiguous run of indices, and tile_of walks tiles in groups of `group_m` tile-rows
+// (column-major inside a group) for operand reuse in L2.
+__device__ __forceinline__ int xcd_contiguous(int pid, int nwg, int nxcd) {
+  if (nxcd <= 1) return pid;
+  int xcd = pid % nxcd, loc = pid / nxcd;
+  int per = nwg / nxcd, rem = nwg % nxcd;
   return xcd * per + (xcd < rem ? xcd : rem) + loc;
 }
 __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
@@ -73,9 +75,9 @@ __device__ __forceinline__ void tile_of_grouped(int t, int tiles_m, int tiles_n,
   tm = by_columns ? minor : major;
   tn = by_columns ? major : minor;
 }
-__device__ __forceinline__ void map_tile(int pid, int nwg, int tiles_m, int tiles_n, int group_m,
+__device__ __forceinline__ void map_tile(int pid, int nwg, int nxcd, int tiles_m, int tiles_n, int group_m,
                                          int& tm, int& tn) {
-  tile_of_grouped(xcd_contiguous(pid, nwg), tiles_m, tiles_n, group_m, tm, tn);
+  tile_of_grouped(xcd_contiguous(pid, nwg, nxcd), tiles_m, tiles_n, group_m, tm, tn);
 }
 
 template <int BK>
@@ -180,7 +182,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
 
   const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
   int tm_i, tn_i;
-  map_tile(blockIdx.x, gridDim.x, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  map_tile(blockIdx.x, gridDim.x, ga.nxcd, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
   const int m0 = tm_i * BM, n0 = tn_i * BN;
 
   f32x16 acc[NB][TM][TN];

@@ -116,7 +116,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
   // Workgroup -> (split, tile): all tiles of split 0, then all tiles of split 1, ...
   const int ntiles = tiles_m * tiles_n;
-  const int u = xcd_contiguous(pid, nwg);
+  const int u = xcd_contiguous(pid, nwg, ga.nxcd);
   const int split = Epi::SPLIT ? u / ntiles : 0;
   int tm_i, tn_i;
   tile_of_grouped(u - split * ntiles, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
@@ -497,9 +497,8 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
           typename Epi>
 hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
-  auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  static LdsAttrOnce lds_attr;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES, lds_attr)) return e;
+  constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
+  if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   const int splits = Epi::SPLIT ? ga.splits : 1;
   dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN) * splits), block(Cfg::NW * 64);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
@@ -510,9 +509,8 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
           typename Epi>
 hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
-  auto kern = gemm_group_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
-  static LdsAttrOnce lds_attr;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES, lds_attr)) return e;
+  constexpr auto kern = gemm_group_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
+  if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   int total = 0;
   for (int g = 0; g < grp.count; ++g) {
     grp.first[g] = total;

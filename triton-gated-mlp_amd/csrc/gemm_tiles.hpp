@@ -85,20 +85,32 @@ struct LdsTile {
   }
 };
 
-// Raises the dynamic-LDS limit of `kernel` (needed above 64 KiB) the first time the kernel is
-// launched on a device; the attribute is per device and per kernel, so every launch site keeps a
-// flag array of its own.  After the first launch no runtime call but hipGetDevice is made, which
-// also keeps the launch path free of attribute calls while a stream is being captured.
-struct LdsAttrOnce {
-  std::atomic<unsigned char> done[64];
+// Kernels with more than 64 KiB of dynamic LDS need the limit raised per device and per kernel
+// (hipFuncSetAttribute), a call that must not be made while a stream is being captured.  Every
+// such kernel has one LdsKernel object, registered when the library is loaded: prepare_lds_kernels
+// (called by gmlp_init) raises the limit of all of them on the current device up front; a launch
+// that still finds its kernel unprepared does it itself unless its stream is capturing, in which
+// case it reports hipErrorStreamCaptureUnsupported instead of making the call.
+struct LdsKernel {
+  const void* kernel;
+  int bytes;
+  std::atomic<unsigned char> done[64];  // per device
+  LdsKernel(const void* k, int b);      // registers itself (api.hip)
 };
-inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, LdsAttrOnce& once) {
+hipError_t prepare_lds_kernels();  // every registered kernel, on the current device
+template <auto KERNEL, int BYTES>
+inline LdsKernel lds_kernel_of{(const void*)KERNEL, BYTES};
+
+inline hipError_t allow_dynamic_lds(LdsKernel& k, hipStream_t s) {
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   const bool tracked = dev >= 0 && dev < 64;
-  if (tracked && once.done[dev].load(std::memory_order_acquire)) return hipSuccess;
-  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes)) return e;
-  if (tracked) once.done[dev].store(1, std::memory_order_release);
+  if (tracked && k.done[dev].load(std::memory_order_acquire)) return hipSuccess;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipError_t e = hipStreamIsCapturing(s, &st)) return e;
+  if (st != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
+  if (hipError_t e = hipFuncSetAttribute(k.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, k.bytes)) return e;
+  if (tracked) k.done[dev].store(1, std::memory_order_release);
   return hipSuccess;
 }
 

@@ -38,9 +38,8 @@ template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KS, bool 
           bool EDGE, typename Epi>
 hipError_t launch_gemm(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
   typedef GemmConfig<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE> Cfg;
-  auto kern = gemm_kernel<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE, Epi>;
-  static LdsAttrOnce lds_attr;
-  if (hipError_t e = allow_dynamic_lds((const void*)kern, Cfg::LDS_BYTES, lds_attr)) return e;
+  constexpr auto kern = gemm_kernel<T, BM, BN, BK, WGM, WGN, A_KS, B_KS, NB, EDGE, Epi>;
+  if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
   dim3 grid(tiles_m * tiles_n), block(Cfg::NT);
   hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);

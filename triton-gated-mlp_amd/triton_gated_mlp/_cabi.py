@@ -16,7 +16,7 @@ from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD, GMLP_OP_GATEUP_FWD = 0, 1, 2, 3, 4
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
 # tables (src/triton_gated_mlp/gated_mlp.py:17-37).
@@ -42,6 +42,7 @@ _f32 = ctypes.c_float
 _SIGNATURES = {
     "gmlp_abi_version": (_int, []),
     "gmlp_last_error": (ctypes.c_char_p, []),
+    "gmlp_init": (_int, []),
     "gmlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
     "gmlp_gateup_fwd": (
         _int,

@@ -289,6 +289,14 @@ class FusedGatedMLP(_GatedMLPBase):
                 return _fwd.decode_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, self.act_fn)
             hs = _fwd.gateup_fwd(x2, W_gate, b_gate, W_up, b_up, 0.0, 0, 0, save_activations=False, act_fn=self.act_fn)
             return _fwd.linear_fwd(hs.hidden, W_down, b_down)
+        if x2.is_cuda and torch.cuda.is_current_stream_capturing():
+            # Capturing forward + backward with torch.cuda.graph has ended in a host-side crash inside
+            # the runtime's end-of-capture call on ROCm 7.2; until its cause is known the module
+            # refuses rather than take the process down.  Inference forwards capture fine.
+            raise RuntimeError(
+                "FusedGatedMLP: capturing a step that records an autograd graph (training forward) into a "
+                "HIP graph is not supported; capture inference forwards (torch.no_grad(), eval mode) only"
+            )
         seed, offset = self._next_dropout_state() if p > 0.0 else (0, 0)
         if p > 0.0:
             self.last_dropout_states.append((row0, M, seed, offset))
