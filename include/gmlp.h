@@ -75,7 +75,8 @@ const char* gmlp_last_error(void);
 /*
  * Optional set-up for the current HIP device: makes every one-time runtime call the entry points
  * would otherwise make at their first launch on that device (raising the dynamic-LDS limit of each
- * kernel, reading the compute-unit count).  Call it once per device before capturing a stream into a HIP graph: those
+ * kernel, reading the compute-unit count, resolving the address of the static scratch array of
+ * gmlp_colsum_static).  Call it once per device before capturing a stream into a HIP graph: those
  * calls are not allowed during capture, and an entry point that still needs one while its stream
  * is capturing returns GMLP_EHIP (hipErrorStreamCaptureUnsupported) instead of making it.
  * No counterpart in the reference (Triton compiles and configures its kernels at first launch,
@@ -177,6 +178,21 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
  */
 int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C, int dtype,
                 void* stream);
+
+/*
+ * gmlp_colsum for callers that cannot allocate device memory (code running under HIP graph capture,
+ * serving loops and harnesses that forbid allocation): the same kernels and the same result, bit
+ * for bit, with the first stage's partial sums kept in a static device array of the library instead
+ * of a caller's workspace.  It has no counterpart in the reference.  The array holds
+ * 64 x GMLP_COLSUM_STATIC_MAX_C floats (8 MiB) on every GPU the library has run on, until the
+ * process ends; C beyond GMLP_COLSUM_STATIC_MAX_C is rejected with GMLP_ESHAPE.  The call makes no
+ * hipMalloc/hipFree.  Every call on a GPU uses that GPU's one array: calls that may overlap on one
+ * GPU (different streams, or graphs replayed concurrently) race and must be serialised by the
+ * caller; calls on one stream are ordered.  Nothing has to be cleared between calls: the first
+ * stage overwrites every partial sum the second stage reads.
+ */
+#define GMLP_COLSUM_STATIC_MAX_C 32768
+int gmlp_colsum_static(const void* a, void* out, int64_t M, int64_t C, int dtype, void* stream);
 
 /*
  * Up to 3 bias gradients of one backward pass in one pair of launches: out[i][C[i]] = Σ_m a[i][m,C[i]].

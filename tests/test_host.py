@@ -73,6 +73,10 @@ def test_argument_validation_returns_codes_without_touching_the_device():
         (lib.gmlp_colsum, (a, a, None, 8, 8, 0, None)),
     ]:
         assert fn(*args) == -1
+    # the entry point without a workspace rejects more columns than its static array holds
+    assert lib.gmlp_colsum_static(a, a, 8, 32768 + 8, 0, None) == -2 and "32768" in err()
+    assert lib.gmlp_colsum_static(a, None, 8, 64, 0, None) == -1
+    assert lib.gmlp_colsum_static(a, a, 8, 12, 0, None) == -2
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, 100, 0, 64, 0) == 64 * 64 * 4
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DECODE_FWD, 16, 8192, 28672, 0) == 0
     # split reduction: asked for by short batches with a long reduction only, never for float32

@@ -39,6 +39,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
   if ((a) < 0 || (a) >= gmlp::ACT_COUNT)                                            \
   return fail(GMLP_EINVAL, "%s: act %d is not one of the GMLP_ACT_* codes", __func__, (int)(a))
 
+static_assert(GMLP_COLSUM_STATIC_MAX_C == gmlp::COLSUM_STATIC_MAX_C, "public limit of gmlp_colsum_static");
 static_assert((int)GMLP_ACT_SILU == (int)gmlp::ACT_SILU && (int)GMLP_ACT_GELU == (int)gmlp::ACT_GELU &&
                   (int)GMLP_ACT_RELU == (int)gmlp::ACT_RELU && (int)GMLP_ACT_LEAKY_RELU == (int)gmlp::ACT_LEAKY_RELU &&
                   (int)GMLP_ACT_SIGMOID == (int)gmlp::ACT_SIGMOID && (int)GMLP_ACT_TANH == (int)gmlp::ACT_TANH &&
@@ -222,7 +223,9 @@ const char* gmlp_last_error(void) { return g_err; }
 
 int gmlp_init(void) {
   (void)num_cu();
-  return hip_result(__func__, gmlp::prepare_lds_kernels());
+  if (hipError_t e = gmlp::prepare_lds_kernels()) return hip_result(__func__, e);
+  float* scratch = nullptr;
+  return hip_result(__func__, gmlp::colsum_static_scratch(&scratch));
 }
 
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {
@@ -584,6 +587,24 @@ int gmlp_colsum(const void* a, void* out, void* workspace, int64_t M, int64_t C,
   const void* as[1] = {a};
   void* outs[1] = {out};
   return gmlp_colsum_grouped(1, as, outs, workspace, M, &C, dtype, stream);
+}
+
+int gmlp_colsum_static(const void* a, void* out, int64_t M, int64_t C, int dtype, void* stream) {
+  using namespace gmlp;
+  GMLP_REQUIRE_PTR(a); GMLP_REQUIRE_PTR(out);
+  GMLP_REQUIRE_DTYPE(dtype);
+  if (int rc = check_dims(__func__, M, 8, C)) return rc;
+  if (int rc = check_mult8(__func__, "C", C)) return rc;
+  if (C > COLSUM_STATIC_MAX_C)
+    return fail(GMLP_ESHAPE, "%s: C = %lld exceeds the %lld columns the library's static scratch array holds "
+                "(use gmlp_colsum with a workspace)", __func__, (long long)C, (long long)COLSUM_STATIC_MAX_C);
+  GMLP_REQUIRE_ALIGNED(a); GMLP_REQUIRE_ALIGNED(out);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = by_dtype(dtype, [&](auto tag) {
+    typedef decltype(tag) T;
+    return launch_colsum_static<T>((const T*)a, (T*)out, M, C, s);
+  });
+  return hip_result(__func__, e);
 }
 
 int gmlp_colsum_grouped(int count, const void* const* a, void* const* out, void* workspace, int64_t M,

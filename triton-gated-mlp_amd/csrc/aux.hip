@@ -150,6 +150,47 @@ template hipError_t launch_colsum_group<f16>(const ColsumGroup<f16>&, int, int64
 template hipError_t launch_colsum_group<bf16>(const ColsumGroup<bf16>&, int, int64_t, hipStream_t);
 template hipError_t launch_colsum_group<float>(const ColsumGroup<float>&, int, int64_t, hipStream_t);
 
+// Column sums for callers that cannot allocate: the partial sums of the first stage live in this
+// array instead of a caller's workspace.  Every GPU the library runs on holds its own copy, at
+// its own address, until the process ends (COLSUM_SPLITS x COLSUM_STATIC_MAX_C floats = 8 MiB).
+// The name below is a host-side handle, not a device address: host code only ever uses the
+// pointer hipGetSymbolAddress returned for the current device.
+static __device__ __align__(256) float scratch[(size_t)COLSUM_SPLITS * COLSUM_STATIC_MAX_C];
+
+hipError_t colsum_static_scratch(float** out) {
+  static std::atomic<float*> known[64];  // per device
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const bool tracked = dev >= 0 && dev < 64;
+  float* p = tracked ? known[dev].load(std::memory_order_acquire) : nullptr;
+  if (p == nullptr) {
+    void* q = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch))) return e;
+    if (q == nullptr) return hipErrorInvalidSymbol;
+    p = (float*)q;
+    if (tracked) known[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return hipSuccess;
+}
+
+// The first stage writes every partial sum the second stage reads (all COLSUM_SPLITS row ranges of
+// all C columns, zeros for empty ranges), so nothing in the array has to be cleared between calls.
+template <typename T>
+hipError_t launch_colsum_static(const T* a, T* out, int64_t M, int64_t C, hipStream_t s) {
+  float* ws = nullptr;
+  if (hipError_t e = colsum_static_scratch(&ws)) return e;
+  ColsumGroup<T> g = {};
+  g.a[0] = a;
+  g.out[0] = out;
+  g.ws[0] = ws;
+  g.C[0] = C;
+  return launch_colsum_group<T>(g, 1, M, s);
+}
+template hipError_t launch_colsum_static<f16>(const f16*, f16*, int64_t, int64_t, hipStream_t);
+template hipError_t launch_colsum_static<bf16>(const bf16*, bf16*, int64_t, int64_t, hipStream_t);
+template hipError_t launch_colsum_static<float>(const float*, float*, int64_t, int64_t, hipStream_t);
+
 __global__ void __launch_bounds__(256)
     dropout_mask_kernel(uint8_t* __restrict__ mask, size_t n4, DropoutParams d) {
   size_t stride = (size_t)gridDim.x * blockDim.x;

@@ -87,6 +87,12 @@ struct ColsumGroup {
 template <typename T>
 hipError_t launch_colsum_group(const ColsumGroup<T>& g, int count, int64_t M, hipStream_t s);
 size_t colsum_workspace_bytes(int64_t M, int64_t C);
+// Column sums of one array with the first stage's partial sums in a static device array of the
+// library (no workspace argument, no allocation); C <= COLSUM_STATIC_MAX_C.
+constexpr int64_t COLSUM_STATIC_MAX_C = 32768;
+hipError_t colsum_static_scratch(float** out);  // address of that array on the current device
+template <typename T>
+hipError_t launch_colsum_static(const T* a, T* out, int64_t M, int64_t C, hipStream_t s);
 hipError_t launch_dropout_mask(uint8_t* mask, int64_t M, int64_t N, const DropoutParams& d,
                                hipStream_t s);
 

@@ -55,6 +55,7 @@ _SIGNATURES = {
     "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr]),
     "gmlp_dw_bwd_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _c_ptr, _int, _c_ptr]),
     "gmlp_colsum": (_int, [_c_ptr] * 3 + [_i64, _i64, _int, _c_ptr]),
+    "gmlp_colsum_static": (_int, [_c_ptr] * 2 + [_i64, _i64, _int, _c_ptr]),
     "gmlp_colsum_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _int, _c_ptr]),
     "gmlp_decode_fwd": (_int, [_c_ptr] * 10 + [_i64, _i64, _i64, _int, _int, _c_ptr]),
     "gmlp_dropout_mask": (_int, [_c_ptr, _i64, _i64, _f32, _u64, _u64, _c_ptr]),

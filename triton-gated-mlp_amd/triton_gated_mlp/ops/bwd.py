@@ -177,6 +177,29 @@ def colsum(a: Tensor) -> Tensor:
     return out
 
 
+def colsum_static(a: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    """colsum through the entry point that allocates nothing (gmlp_colsum_static): the partial sums
+    live in a static device array of the library, so only `out` is the caller's (pass one to make
+    the call allocation-free, e.g. under graph capture).  At most 32768 columns; calls that overlap
+    on one GPU share the array and race."""
+    if a.ndim != 2 or a.shape[0] < 1:
+        raise ValueError("colsum_static takes a 2-D tensor with at least one row")
+    dev = _cabi.require_gpu(a, out)
+    code = _cabi.dtype_code(a.dtype)
+    if not a.is_contiguous():
+        raise ValueError("colsum_static takes a contiguous tensor (it would have to allocate a copy)")
+    M, C = a.shape
+    if out is None:
+        out = torch.empty((C,), dtype=a.dtype, device=dev)
+    elif tuple(out.shape) != (C,) or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor of C elements")
+    with torch.cuda.device(dev):
+        _cabi.check(
+            _cabi.lib().gmlp_colsum_static(_cabi.ptr(a), _cabi.ptr(out), M, C, code, _cabi.stream_ptr(dev))
+        )
+    return out
+
+
 def colsum_grouped(arrays):
     """[Σ_m a[m,:] for a in arrays] (at most 3 arrays with the same number of rows) in one pair of
     launches: the bias gradients of one backward pass."""
