@@ -62,7 +62,11 @@ struct Traits<float> {
 
 // sigma(x) = 1/(1+e^-x), silu(x) = x*sigma(x), silu'(x) = sigma*(1 + x*(1-sigma)); all fp32.
 // Same forms as the reference's _compute_sigma/_silu_fwd/_silu_bwd (src/triton_gated_mlp/ops/act.py:28-45).
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// Reciprocals are the hardware's v_rcp_f32 (1 ulp): a plain `1.0f / y` compiles to the IEEE division
+// sequence of eleven instructions, which made the activation arithmetic the longest part of the
+// fused epilogues.
+__device__ __forceinline__ float rcp_f32(float y) { return __builtin_amdgcn_rcpf(y); }
+__device__ __forceinline__ float sigmoid_f32(float x) { return rcp_f32(1.0f + __expf(-x)); }
 __device__ __forceinline__ float silu_f32(float x) { return x * sigmoid_f32(x); }
 __device__ __forceinline__ float silu_grad_f32(float x) {
   float s = sigmoid_f32(x);
@@ -79,7 +83,7 @@ struct NormalCdf {
 };
 __device__ __forceinline__ NormalCdf normal_cdf_f32(float x) {
   const float ax = fabsf(x);
-  const float t = 1.0f / (1.0f + 0.23164189f * ax);  // p / sqrt 2, p = 0.3275911
+  const float t = rcp_f32(1.0f + 0.23164189f * ax);  // p / sqrt 2, p = 0.3275911
   const float e = __expf(-0.5f * x * x);
   float poly = 1.061405429f;
   poly = poly * t - 1.453152027f;
@@ -94,7 +98,7 @@ __device__ __forceinline__ NormalCdf normal_cdf_f32(float x) {
 __device__ __forceinline__ float tanh_f32(float x) {
   const float ax = fabsf(x), x2 = x * x;
   const float e = __expf(-2.0f * ax);
-  const float big = (1.0f - e) / (1.0f + e);
+  const float big = (1.0f - e) * rcp_f32(1.0f + e);
   const float small = ax * (1.0f + x2 * (-0.33333333f + x2 * (0.13333333f - x2 * 0.053968254f)));
   return copysignf(ax < 0.25f ? small : big, x);
 }

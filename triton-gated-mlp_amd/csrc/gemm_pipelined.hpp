@@ -329,14 +329,24 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 
   int kt = kt_first;
   for (; kt + 1 < kt_total; ++kt) tile_body(kt, std::true_type{});
+  // (the operand fragments are still live during the last reduction tile: the first PD_EARLY
+  // items are fetched before it, the rest of the PD behind it)
+  constexpr int PD_EARLY = PD < 8 ? PD : 8;
 #pragma unroll
-  for (int q = 0; q < PD; ++q) {
+  for (int q = 0; q < PD_EARLY; ++q) {
     int row, m, n, cg;
     item_pos(q, row, m, n, cg);
     Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
   }
   tile_body(kt, std::false_type{});
-  wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
+#pragma unroll
+  for (int q = PD_EARLY; q < PD; ++q) {
+    int row, m, n, cg;
+    item_pos(q, row, m, n, cg);
+    Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
+  }
+  if constexpr (PD == PD_EARLY) wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
+  else wait_vmem<2 * (PD - PD_EARLY)>();
 
   // ---- epilogue: transpose MI-row slabs through LDS, after which each lane owns 8 consecutive
   // columns of one row: the fp32 accumulators themselves, with the arithmetic behind the transpose
@@ -379,12 +389,22 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           *(f32x4*)v1 = *(const f32x4*)p1;
           *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
         }
+#ifdef GMLP_PREFETCH_FIRST
+        const typename Epi::template Prefetch<8> cur = pf[q % (PD > 0 ? PD : 1)];
+        if (q + PD < NITEMS) {
+          int row2, m2, n2, cg2;
+          item_pos(q + PD, row2, m2, n2, cg2);
+          Epi::template prefetch<8>(ea, min(m2, ga.M - 1), min(n2, ga.N - 8), pf[q % (PD > 0 ? PD : 1)]);
+        }
+        if (m < ga.M && n < ga.N) Epi::template apply<8, ACT>(ea, m, n, v0, v1, cur);
+#else
         if (m < ga.M && n < ga.N) Epi::template apply<8, ACT>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
         if (q + PD < NITEMS) {
           int row2, m2, n2, cg2;
           item_pos(q + PD, row2, m2, n2, cg2);
           Epi::template prefetch<8>(ea, min(m2, ga.M - 1), min(n2, ga.N - 8), pf[q % (PD > 0 ? PD : 1)]);
         }
+#endif
       }
     }
   };
