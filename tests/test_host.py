@@ -309,3 +309,23 @@ def test_async_load_checker_flags_registers_touched_before_their_wait(tmp_path):
         "\ts_endpgm\n"
     )
     assert mod.check(str(bad)) == 1
+
+
+def test_m0_checker_flags_compiler_generated_m0_uses(tmp_path):
+    """csrc/check_m0.py (run on every GEMM unit by the build): M0 written inside the inline-assembly
+    blocks is the kernels' own; a write or an implied use outside them, in a kernel that holds
+    global->LDS loads, fails the build.  Kernels without such loads are not its business."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("check_m0", ROOT / "triton-gated-mlp_amd" / "csrc" / "check_m0.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    dma = "\t;;#ASMSTART\n\ts_mov_b32 m0, s4\n\ts_nop 0\n\t;;#ASMEND\n\t;;#ASMSTART\n\tbuffer_load_dwordx4 v1, s[8:11], s2 offen offset:1024 lds\n\t;;#ASMEND\n"
+    good = "_Z4kern:\n" + dma + "\tv_mfma_f32_16x16x32_f16 a[0:3], v[0:3], v[4:7], a[0:3]\n\ts_endpgm\n"
+    bad_write = "_Z4kern:\n" + dma + "\ts_mov_b32 m0, s9\n\ts_endpgm\n"
+    bad_use = "_Z4kern:\n" + dma + "\tv_movrels_b32_e32 v0, v1\n\ts_endpgm\n"
+    other = "_Z5plain:\n\ts_mov_b32 m0, s9\n\ts_endpgm\n"
+    for text, expect in ((good, 0), (bad_write, 1), (bad_use, 1), (other, 0), (good + other, 0), (other + bad_write, 1)):
+        f = tmp_path / "k.s"
+        f.write_text(text)
+        assert mod.check(str(f)) == expect

@@ -49,8 +49,12 @@ __device__ __forceinline__ void load16_to_lds(buffer_rsrc r, uint32_t voffset, u
 // written once for up to four loads, which then differ by the instruction's immediate offset
 // (0, 1024, 2048 or 3072).  The immediate is added to the LDS address AND to the global address,
 // so the caller passes a voffset that already has it subtracted (see DMA_BIAS in gemm_pipelined.hpp).
-// The compiler is not told that M0 stays live between the two statements; it has no use for M0 of
-// its own in kernels without indirect register indexing, message or GWS instructions.
+// That M0 must stay live until the group's last load cannot be expressed to the compiler (M0 is a
+// reserved register: it is not accepted as an operand, and not reliably as a clobber), which has no
+// use for M0 of its own in kernels without indirect register
+// indexing, message or GWS instructions.  The build does not take that on trust: csrc/check_m0.py
+// scans the device assembly of every GEMM unit and fails it if any instruction outside the
+// inline-assembly blocks writes or implies M0 in a kernel that contains these loads.
 __device__ __forceinline__ void set_lds_dma_base(uint32_t lds_wave_base) {
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
