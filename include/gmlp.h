@@ -66,7 +66,10 @@ enum gmlp_op {
   GMLP_OP_COLSUM = 1,
   GMLP_OP_LINEAR_FWD = 2,
   GMLP_OP_DX_BWD = 3,
-  GMLP_OP_GATEUP_FWD = 4
+  GMLP_OP_GATEUP_FWD = 4,
+  GMLP_OP_DH_BWD = 5,
+  GMLP_OP_DW_BWD = 6,
+  GMLP_OP_DW_BWD_GROUPED = 7
 };
 
 int gmlp_abi_version(void);
@@ -88,7 +91,16 @@ int gmlp_init(void);
  * Workspace bytes the caller must provide for `op` at the given problem size (0 if none), with
  * (M, K, N) as the entry point of that name takes them: GMLP_OP_COLSUM (M, 0, C),
  * GMLP_OP_LINEAR_FWD (M, R, C), GMLP_OP_DX_BWD (M, K, N), GMLP_OP_GATEUP_FWD (M, K, N),
- * GMLP_OP_DECODE_FWD (M, K, N).
+ * GMLP_OP_DECODE_FWD (M, K, N), GMLP_OP_DH_BWD (M, K, N), GMLP_OP_DW_BWD (Mred, R, C),
+ * GMLP_OP_DW_BWD_GROUPED (arguments ignored: an upper bound for any set of problems, 128 MiB on a
+ * whole MI355X).  The values are enumerators, not flags: ask per operation; one buffer of the
+ * largest answer serves every call of a forward or backward pass (calls on one stream are ordered).
+ * Two things use a workspace, and without one (NULL, 0) every entry point computes the same result
+ * more slowly on the shapes concerned: split reductions for short batches (see gmlp_linear_fwd),
+ * and stream-K for grids of large tiles that end in a thinly filled round of workgroups while the
+ * reduction is long (the last round's tiles are then shared out by reduction range over all compute
+ * units, fp32 partial sums pass through the workspace and a second launch adds them up in a fixed
+ * order: results do not depend on timing).
  */
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype);
 
@@ -127,10 +139,11 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
  * Replaces the autograd backward of down_proj plus _compute_quantities_for_bwd
  * (src/triton_gated_mlp/ops/bwd.py:89-211; closed form in gated_mlp.py:131-144).  g, u are the
  * tensors written by gmlp_gateup_fwd (g_save, u_save).  dg, du are [M,N].
+ * workspace (may be NULL): gmlp_workspace_bytes(GMLP_OP_DH_BWD, M, K, N, dtype) bytes.
  */
 int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
                 int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p, uint64_t seed,
-                uint64_t offset, void* stream);
+                uint64_t offset, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Element-wise gating backward for callers that already hold dH (the reference's operator-level
@@ -156,9 +169,10 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
  * Replaces _compute_dW_up_dW_gp (src/triton_gated_mlp/ops/bwd.py:386-463; gated_mlp.py:152-155)
  * with (lhs,rhs) = (dG,x), (dU,x); and the autograd dW of down_proj with (lhs,rhs) = (dY,H).
  * Requires R % 8 == 0, C % 8 == 0.
+ * workspace (may be NULL): gmlp_workspace_bytes(GMLP_OP_DW_BWD, Mred, R, C, dtype) bytes.
  */
 int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_t R, int64_t C,
-                int dtype, void* stream);
+                int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Up to 3 weight gradients that share the reduction length Mred, enqueued as ONE grid when every
@@ -166,9 +180,14 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
  *   dw[i][R[i],C[i]] = lhs[i][Mred,R[i]]ᵀ · rhs[i][Mred,C[i]],  i < count.
  * Same reference counterparts as gmlp_dw_bwd; one launch for dW_gate, dW_up and dW_down avoids
  * three partially filled last rounds of workgroups.
+ * workspace (may be NULL): gmlp_dw_bwd_grouped_workspace_bytes(count, Mred, R, C, dtype) bytes (what
+ * this set of problems uses, often 0), or the bound gmlp_workspace_bytes(GMLP_OP_DW_BWD_GROUPED, ...).
  */
+size_t gmlp_dw_bwd_grouped_workspace_bytes(int count, int64_t Mred, const int64_t* R, const int64_t* C,
+                                           int dtype);
 int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rhs, void* const* dw,
-                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* stream);
+                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream);
 
 /*
  * Bias gradient: out[C] = Σ_m a[m,C], fp32 accumulation in a fixed order (deterministic).

@@ -764,6 +764,100 @@ def test_benchmark_sweep_reports_both_providers_and_step_memory():
         assert kept_mb <= rm["fused"] < 40 * kept_mb, f"fused step peak {rm['fused']:.2f} MB at {s}"
 
 
+def _streamk_expected(op, M, K, N, code=0):
+    from triton_gated_mlp import _cabi
+
+    return _cabi.lib().gmlp_workspace_bytes(op, M, K, N, code)
+
+
+def test_streamk_seams_every_gemm_kind_against_fp32_matmul():
+    """Grids of large tiles that end in a thinly filled round with a long reduction run their last
+    round's tiles as stream-K pieces (several workgroups per tile, fp32 partial sums through the
+    workspace, a second launch adds them up in a fixed order).  Every kind of GEMM of the MLP on a
+    shape that takes that path (the workspace query says so), against fp32 products of the same
+    rounded operands; twice, bit-identical (no dependence on timing)."""
+    from triton_gated_mlp import _cabi
+    from triton_gated_mlp.ops import bwd as ops_bwd
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(17)
+    rnd = lambda *shape, s=1.0: (s * torch.randn(*shape, generator=g)).half()
+    f = lambda t: t.float()
+
+    # down projection: out [2048, 11264] = 352 tiles (1.375 rounds), reduction 5184 = 81 tiles; 96 tiles
+    # over 256 workgroups: ranges that straddle tiles (the other cases below cut every tile into a
+    # whole number of pieces)
+    M, R, C = 2048, 5184, 11264
+    assert _streamk_expected(_cabi.GMLP_OP_LINEAR_FWD, M, R, C) == (96 + 256) * 65536 * 4
+    a, w, b = rnd(M, R), rnd(C, R, s=0.02), rnd(C, s=0.1)
+    y = ops_fwd.linear_fwd(a.to(dev), w.to(dev), b.to(dev))
+    assert torch.equal(y, ops_fwd.linear_fwd(a.to(dev), w.to(dev), b.to(dev)))
+    _close("linear stream-K", y, f(a) @ f(w).T + f(b))
+    # the same call without a workspace (one workgroup per tile throughout): same values up to the
+    # order of the fp32 additions in the shared-out tiles
+    y0 = torch.empty_like(y)
+    ad, wd, bd = a.to(dev), w.to(dev), b.to(dev)
+    _cabi.check(_cabi.lib().gmlp_linear_fwd(ad.data_ptr(), wd.data_ptr(), bd.data_ptr(), y0.data_ptr(), M, R, C, 0, None, 0,
+                                            _cabi.stream_ptr(dev)))
+    torch.cuda.synchronize()
+    assert (y.float() - y0.float()).abs().max().item() <= 2e-3 * y0.float().abs().max().item()
+    assert not torch.equal(y, torch.zeros_like(y))
+
+    # gate/up: [2048, 5120] hidden = 8 x 40 tiles of 256 x 128, reduction 4352; biases, dropout, G and U kept
+    M, K, N = 2048, 4352, 5120
+    assert _streamk_expected(_cabi.GMLP_OP_GATEUP_FWD, M, K, N) > 0
+    x, wg, wu, bg, bu = rnd(M, K), rnd(N, K, s=0.02), rnd(N, K, s=0.02), rnd(N, s=0.1), rnd(N, s=0.1)
+    p, seed = 0.25, 4242
+    hs = ops_fwd.gateup_fwd(x.to(dev), wg.to(dev), bg.to(dev), wu.to(dev), bu.to(dev), p, seed, 3, save_activations=True)
+    hs2 = ops_fwd.gateup_fwd(x.to(dev), wg.to(dev), bg.to(dev), wu.to(dev), bu.to(dev), p, seed, 3, save_activations=True)
+    assert torch.equal(hs.hidden, hs2.hidden) and torch.equal(hs.gate, hs2.gate) and torch.equal(hs.up, hs2.up)
+    keep = torch.from_numpy(philox.keep_mask(M, N, p, seed, 3))
+    ref = oracle.hidden_forward(f(x), f(wg), f(bg), f(wu), f(bu), keep, p)
+    _close("gate/up stream-K H", hs.hidden, ref["H"])
+    _close("gate/up stream-K G", hs.gate, ref["G"])
+    _close("gate/up stream-K U", hs.up, ref["U"])
+
+    # dH with the gating epilogue: [2048, 10240] = 320 tiles, reduction 4352
+    M, K, N = 2048, 4352, 10240
+    assert _streamk_expected(_cabi.GMLP_OP_DH_BWD, M, K, N) > 0
+    dy, wdn, G, U = rnd(M, K), rnd(K, N, s=0.02), rnd(M, N), rnd(M, N)
+    dg, du = ops_bwd.dh_bwd(dy.to(dev), wdn.to(dev), G.to(dev), U.to(dev), p, seed, 5)
+    dg2, du2 = ops_bwd.dh_bwd(dy.to(dev), wdn.to(dev), G.to(dev), U.to(dev), p, seed, 5)
+    assert torch.equal(dg, dg2) and torch.equal(du, du2)
+    keep = torch.from_numpy(philox.keep_mask(M, N, p, seed, 5))
+    hb = oracle.hidden_backward(f(dy) @ f(wdn), f(G), f(U), keep, p)
+    _close("dH stream-K dG", dg, hb["dG"])
+    _close("dH stream-K dU", du, hb["dU"])
+
+    # dX: [2048, 10240] = 320 tiles, two reduction segments of 2176 = 68 tiles together
+    M, K, N = 2048, 10240, 2176
+    assert _streamk_expected(_cabi.GMLP_OP_DX_BWD, M, K, N) > 0
+    dgv, duv, wg, wu = rnd(M, N), rnd(M, N), rnd(N, K, s=0.02), rnd(N, K, s=0.02)
+    dx = ops_bwd.dx_bwd(dgv.to(dev), duv.to(dev), wg.to(dev), wu.to(dev))
+    assert torch.equal(dx, ops_bwd.dx_bwd(dgv.to(dev), duv.to(dev), wg.to(dev), wu.to(dev)))
+    _close("dX stream-K", dx, f(dgv) @ f(wg) + f(duv) @ f(wu))
+
+    # dW, one problem: [10240, 2048] = 320 tiles, reduction over 4360 token rows (not a multiple of 64)
+    Mred, R, C = 4360, 10240, 2048
+    assert _streamk_expected(_cabi.GMLP_OP_DW_BWD, Mred, R, C) > 0
+    lhs, rhs = rnd(Mred, R), rnd(Mred, C)
+    dw = ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev))
+    assert torch.equal(dw, ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev)))
+    _close("dW stream-K", dw, f(lhs).T @ f(rhs), atol=ATOL * 40)
+
+    # dW, grouped: 64 + 64 + 256 = 384 tiles (1.5 rounds); the shared-out tiles are the last 128 of
+    # the last problem (reduction of 102 tiles: half a round saved is worth the second launch)
+    Mred = 6528
+    pairs = [(rnd(Mred, 2048), rnd(Mred, 2048)), (rnd(Mred, 2048), rnd(Mred, 2048)), (rnd(Mred, 4096), rnd(Mred, 4096))]
+    dev_pairs = [(a_.to(dev), b_.to(dev)) for a_, b_ in pairs]
+    outs = ops_bwd.dw_bwd_grouped(dev_pairs)
+    outs2 = ops_bwd.dw_bwd_grouped(dev_pairs)
+    for (a_, b_), got, again in zip(pairs, outs, outs2):
+        assert torch.equal(got, again)
+        _close("dW grouped stream-K", got, f(a_).T @ f(b_), atol=ATOL * 40)
+
+
 def test_grouped_weight_gradients_equal_single_launches():
     """gmlp_dw_bwd_grouped (one grid) is bit-identical to three gmlp_dw_bwd launches."""
     from triton_gated_mlp.ops import bwd as ops_bwd
@@ -779,7 +873,7 @@ def test_grouped_weight_gradients_equal_single_launches():
         pairs = [(dg, x), (du, x), (dy, h)]
         grouped = ops_bwd.dw_bwd_grouped(pairs)
         for (a, b), got in zip(pairs, grouped):
-            assert torch.equal(got, ops_bwd.dw_bwd(a, b))
+            assert torch.equal(got, ops_bwd.dw_bwd(a, b))  # (neither form shares out tiles at these shapes)
         _close("dW_gate grouped", grouped[0], dg.float().cpu().T @ x.float().cpu(), atol=ATOL * 40)
 
 

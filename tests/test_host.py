@@ -66,10 +66,10 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 40, 256, 0, 0, None) == -2
     assert lib.gmlp_decode_fwd(a, a, a, a, None, None, None, a, a, None, 16, 256, 128, 0, 0, None) == -2
     for fn, args in [
-        (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0, 0.0, 0, 0, None)),
+        (lib.gmlp_dh_bwd, (a, a, a, None, a, a, 8, 8, 8, 0, 0, 0.0, 0, 0, None, 0, None)),
         (lib.gmlp_gating_bwd, (a, a, a, a, None, 8, 8, 0, 0, 0.0, 0, 0, None)),
         (lib.gmlp_dx_bwd, (a, a, a, a, None, 8, 8, 8, 0, None, 0, None)),
-        (lib.gmlp_dw_bwd, (a, None, a, 8, 8, 8, 0, None)),
+        (lib.gmlp_dw_bwd, (a, None, a, 8, 8, 8, 0, None, 0, None)),
         (lib.gmlp_colsum, (a, a, None, 8, 8, 0, None)),
     ]:
         assert fn(*args) == -1
@@ -92,6 +92,15 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert n > 0 and n % (2 * 64 * 13824 * 4) == 0
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, 64, 8192, 28672, 0) == 0
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_GATEUP_FWD, 8192, 4096, 14336, 0) == 0
+    # stream-K: asked for by grids of large tiles that end in a thinly filled round while the
+    # reduction is long (256 compute units assumed without a GPU): 1.5 rounds of the down
+    # projection share out 128 tiles over 256 workgroups, 384 slots of 256 x 256 floats
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_LINEAR_FWD, 6144, 14336, 4096, 0) == 384 * 65536 * 4
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DW_BWD, 8192, 4096, 14336, 0) == 384 * 65536 * 4  # 3.5 rounds
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DH_BWD, 8192, 4096, 14336, 0) == 0  # 7 whole rounds
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DH_BWD, 2048, 2048, 5632, 1) == 0  # short reduction: not worth it
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DW_BWD_GROUPED, 0, 0, 0, 0) == 512 * 65536 * 4
+    assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DW_BWD_GROUPED, 0, 0, 0, 2) == 0
 
 
 def test_error_codes_map_to_python_exceptions():

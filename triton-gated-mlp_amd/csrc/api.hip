@@ -181,6 +181,49 @@ int64_t whole_round_tile_rows(int dtype, int64_t rows, int64_t cols, int64_t red
   return rounds >= 1 && tail > 0 && 2 * tail <= cus && whole >= 1 && whole < tiles_m ? whole : 0;
 }
 
+// Stream-K plan for a grid of `tiles` large output tiles with `kt` 64-wide reduction tiles each
+// (tiles of all problems of a grouped launch together).  The tiles beyond the last whole round of
+// workgroups (one per compute unit) are shared out by reduction range when that beats running them
+// as a thinly filled round: a round filled to the fraction f costs about 0.6 + 0.4 f of a full one
+// (see pick_tile) against f with stream-K, plus the partial sums' round trip through memory and the
+// second launch (about 45 us, i.e. 30 reduction tiles' time): worth it when (1 - f) * kt > 50.
+// Every stream-K workgroup gets at least 8 reduction tiles.
+struct StreamK {
+  int tiles = 0, wgs = 0, chunks = 0;
+  size_t ws_bytes = 0;
+};
+StreamK plan_streamk(int dtype, int64_t tiles, int64_t kt) {
+  StreamK p;
+  const int64_t cus = num_cu(), tail = tiles % cus;
+  if (dtype == GMLP_F32 || tail == 0 || kt < 8) return p;
+  if ((double)(cus - tail) / (double)cus * (double)kt <= 50.0) return p;
+  int64_t wgs = tail * kt / 8;
+  if (wgs > cus) wgs = cus;
+  if (wgs < 1 || tail * kt >= ((int64_t)1 << 30)) return p;
+  p.tiles = (int)tail;
+  p.wgs = (int)wgs;
+  // A whole number of pieces per tile when that still fills (nearly) all compute units: the
+  // workgroups of an XCD then share operand panels (measured on 128 tiles in halves: the pieces'
+  // launch 123 -> see DESIGN).
+  const int64_t per_tile = wgs / tail;
+  if (per_tile >= 2 && per_tile * tail * 10 >= wgs * 9 && kt / per_tile >= 8) {
+    p.chunks = (int)per_tile;
+    p.wgs = (int)(per_tile * tail);
+  }
+  p.ws_bytes = (size_t)(p.tiles + p.wgs) * 65536 * sizeof(float);  // 256 x 256 accumulators per slot
+  return p;
+}
+// Applies the plan to a launch's arguments when the caller's workspace can hold it.
+bool use_streamk(const StreamK& p, gmlp::GemmArgs& ga, void* workspace, size_t workspace_bytes) {
+  if (p.tiles == 0 || workspace == nullptr || workspace_bytes < p.ws_bytes) return false;
+  ga.sk_tiles = p.tiles;
+  ga.sk_wgs = p.wgs;
+  ga.sk_chunks = p.chunks;
+  ga.sk_ws = (float*)workspace;
+  return true;
+}
+int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
 size_t split_workspace_bytes(int splits, int64_t rows, int64_t cols, int accumulator_sets = 1) {
   return splits > 1 ? (size_t)splits * accumulator_sets * rows * cols * sizeof(float) : 0;
 }
@@ -229,16 +272,35 @@ int gmlp_init(void) {
 }
 
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {
+  // gmlp_dw_bwd_grouped: any set of problems (the plan depends on all of them together): the most
+  // a plan can take, a slot per compute unit for the shared-out tiles and for the workgroups
+  if (op == GMLP_OP_DW_BWD_GROUPED) return dtype == GMLP_F32 ? 0 : (size_t)2 * num_cu() * 65536 * sizeof(float);
   if (M < 1 || N < 1) return 0;
   if (op == GMLP_OP_COLSUM) return gmlp::colsum_workspace_bytes(M, N);
   if (K < 1) return 0;
+  // Each operation asks for the larger of what its split-reduction form (short batches) and its
+  // stream-K form (large tiles whose grid ends in a thinly filled round) would use.
+  auto larger = [](size_t a, size_t b) { return a > b ? a : b; };
+  auto sk = [&](int64_t rows, int64_t cols, int64_t red_tiles, int bn, bool both_ks = false) -> size_t {
+    if (pick_tile(dtype, rows, cols, red_tiles * 64, bn, both_ks) != gmlp::TILE_LARGE) return 0;
+    return plan_streamk(dtype, cdiv(rows, 256) * cdiv(cols, bn), red_tiles).ws_bytes;
+  };
   // gmlp_gateup_fwd(M, K, N): two accumulator sets [M,N], reduction K
   if (op == GMLP_OP_GATEUP_FWD)
-    return split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64, 128), M, N, 2);
+    return larger(split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64, 128), M, N, 2),
+                  K % 64 == 0 ? sk(M, N, K / 64, 128) : 0);
   // gmlp_linear_fwd(M, R = K, C = N): out [M,N], reduction K
-  if (op == GMLP_OP_LINEAR_FWD) return split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64), M, N);
+  if (op == GMLP_OP_LINEAR_FWD)
+    return larger(split_workspace_bytes(pick_splits(dtype, M, N, K, (K + 63) / 64), M, N),
+                  K % 64 == 0 ? sk(M, N, K / 64, 256) : 0);
   // gmlp_dx_bwd(M, K, N): out [M,K], reduction over two segments of N
-  if (op == GMLP_OP_DX_BWD) return split_workspace_bytes(pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64)), M, K);
+  if (op == GMLP_OP_DX_BWD)
+    return larger(split_workspace_bytes(pick_splits(dtype, M, K, N, 2 * ((N + 63) / 64)), M, K),
+                  N % 64 == 0 ? sk(M, K, 2 * (N / 64), 256) : 0);
+  // gmlp_dh_bwd(M, K, N): out [M,N], reduction K
+  if (op == GMLP_OP_DH_BWD) return K % 64 == 0 ? sk(M, N, K / 64, 256) : 0;
+  // gmlp_dw_bwd(Mred = M, R = K, C = N): out [K,N], reduction over the M token rows
+  if (op == GMLP_OP_DW_BWD) return sk(K, N, (M + 63) / 64, 256, true);
   return 0;
 }
 
@@ -266,9 +328,10 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
     typedef decltype(tag) T;
     // The GEMM over output columns [col0, col0 + cols): every per-column pointer moves along, the
     // row pitch of the outputs stays N.
-    auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class) -> hipError_t {
+    auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class, const StreamK* sk = nullptr) -> hipError_t {
       GemmArgs ga = {};
       ga.nxcd = num_xcd();
+      if (sk) use_streamk(*sk, ga, workspace, workspace_bytes);
       ga.A[0] = x; ga.A[1] = x;
       ga.B[0] = (const T*)w_gate + col0 * K; ga.B[1] = (const T*)w_up + col0 * K;
       ga.M = (int)M; ga.N = (int)cols; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)K;
@@ -295,6 +358,9 @@ int gmlp_gateup_fwd(const void* x, const void* w_gate, const void* w_up, const v
     // rounds 114 -> 95 us, 5.375 rounds 627 -> 611 us, 3.5 rounds 416 -> 407 us).
     if (dtype != GMLP_F32 && pick_tile(dtype, M, N, K, 128) == TILE_LARGE) {
       const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 127) / 128, cus = num_cu();
+      // a long reduction: the tiles of the last round are shared out by reduction range instead
+      const StreamK sk = plan_streamk(dtype, tiles_m * tiles_n, K / 64);
+      if (sk.tiles > 0 && workspace != nullptr && workspace_bytes >= sk.ws_bytes) return run(0, N, false, TILE_LARGE, &sk);
       const int64_t rounds = tiles_m * tiles_n / cus, tail = tiles_m * tiles_n % cus;
       const int64_t whole_cols = rounds * cus / tiles_m;  // tile columns of the whole rounds
       if (rounds >= 1 && tail > 0 && 2 * tail <= cus && whole_cols >= 1 && whole_cols < tiles_n) {
@@ -322,9 +388,10 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
     // The GEMM over output columns [col0, col0 + cols); the row pitch of `out` stays C.
-    auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class) -> hipError_t {
+    auto run = [&](int64_t col0, int64_t cols, bool may_split, int force_class, const StreamK* sk = nullptr) -> hipError_t {
       GemmArgs ga = {};
       ga.nxcd = num_xcd();
+      if (sk) use_streamk(*sk, ga, workspace, workspace_bytes);
       ga.A[0] = a; ga.A[1] = a;
       ga.B[0] = (const T*)w + col0 * R; ga.B[1] = ga.B[0];
       ga.M = (int)M; ga.N = (int)cols; ga.K = (int)R; ga.lda = (int)R; ga.ldb = (int)R;
@@ -345,6 +412,8 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
     // gmlp_gateup_fwd)
     if (dtype != GMLP_F32 && pick_tile(dtype, M, C, R, 256) == TILE_LARGE) {
       const int64_t tiles_m = (M + 255) / 256, tiles_n = (C + 255) / 256, cus = num_cu();
+      const StreamK sk = plan_streamk(dtype, tiles_m * tiles_n, R / 64);
+      if (sk.tiles > 0 && workspace != nullptr && workspace_bytes >= sk.ws_bytes) return run(0, C, false, TILE_LARGE, &sk);
       const int64_t rounds = tiles_m * tiles_n / cus, tail = tiles_m * tiles_n % cus;
       const int64_t whole_cols = rounds * cus / tiles_m;
       if (rounds >= 1 && tail > 0 && 2 * tail <= cus && whole_cols >= 1 && whole_cols < tiles_n) {
@@ -359,7 +428,7 @@ int gmlp_linear_fwd(const void* a, const void* w, const void* bias, void* out, i
 
 int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u, void* dg, void* du,
                 int64_t M, int64_t K, int64_t N, int dtype, int act, float dropout_p, uint64_t seed,
-                uint64_t offset, void* stream) {
+                uint64_t offset, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(dy); GMLP_REQUIRE_PTR(w_down); GMLP_REQUIRE_PTR(g); GMLP_REQUIRE_PTR(u);
   GMLP_REQUIRE_PTR(dg); GMLP_REQUIRE_PTR(du);
@@ -372,15 +441,17 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
   if (int rc = check_mult8(__func__, "N", N)) return rc;
   GMLP_REQUIRE_ALIGNED(dy); GMLP_REQUIRE_ALIGNED(w_down); GMLP_REQUIRE_ALIGNED(g);
   GMLP_REQUIRE_ALIGNED(u); GMLP_REQUIRE_ALIGNED(dg); GMLP_REQUIRE_ALIGNED(du);
+  GMLP_REQUIRE_ALIGNED(workspace);
 
   // dH[M,N] = dY[M,K] · W_down[K,N]: reduction over K; B is reduction-strided ([K,N] row-major).
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
     // The GEMM over output rows [row0, row0 + rows): every per-row pointer moves along.
-    auto run = [&](int64_t row0, int64_t rows, int force_class) -> hipError_t {
+    auto run = [&](int64_t row0, int64_t rows, int force_class, const StreamK* sk = nullptr) -> hipError_t {
       GemmArgs ga = {};
       ga.nxcd = num_xcd();
+      if (sk) use_streamk(*sk, ga, workspace, workspace_bytes);
       ga.A[0] = (const T*)dy + row0 * K; ga.A[1] = ga.A[0]; ga.B[0] = w_down; ga.B[1] = w_down;
       ga.M = (int)rows; ga.N = (int)N; ga.K = (int)K; ga.lda = (int)K; ga.ldb = (int)N;
       ga.nseg = 1; ga.group_m = pick_group(rows, N);
@@ -388,6 +459,10 @@ int gmlp_dh_bwd(const void* dy, const void* w_down, const void* g, const void* u
       typename EpiDh<T>::Args ea = {(const T*)g + e0, (const T*)u + e0, (T*)dg + e0, (T*)du + e0, (int)N, act, d, e0};
       return launch_dh<T>(force_class >= 0 ? force_class : pick_tile(dtype, rows, N, K, 256), ga, ea, s);
     };
+    if (dtype != GMLP_F32 && pick_tile(dtype, M, N, K, 256) == TILE_LARGE) {
+      const StreamK sk = plan_streamk(dtype, cdiv(M, 256) * cdiv(N, 256), K / 64);
+      if (sk.tiles > 0 && workspace != nullptr && workspace_bytes >= sk.ws_bytes) return run(0, M, TILE_LARGE, &sk);
+    }
     int64_t whole = whole_round_tile_rows(dtype, M, N, K);
     if (whole > 0) {
       if (hipError_t err = run(0, whole * 256, TILE_LARGE)) return err;
@@ -438,9 +513,10 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
   hipError_t e = by_dtype(dtype, [&](auto tag) -> hipError_t {
     typedef decltype(tag) T;
     // The GEMM over output rows [row0, row0 + rows).
-    auto run = [&](int64_t row0, int64_t rows, bool may_split, int force_class) -> hipError_t {
+    auto run = [&](int64_t row0, int64_t rows, bool may_split, int force_class, const StreamK* sk = nullptr) -> hipError_t {
       GemmArgs ga = {};
       ga.nxcd = num_xcd();
+      if (sk) use_streamk(*sk, ga, workspace, workspace_bytes);
       ga.A[0] = (const T*)dg + row0 * N; ga.A[1] = (const T*)du + row0 * N; ga.B[0] = w_gate; ga.B[1] = w_up;
       ga.M = (int)rows; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
       ga.nseg = 2; ga.group_m = pick_group(rows, K); ga.rotate = rows <= 512;
@@ -456,6 +532,10 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
       }
       return launch_dx<T>(force_class >= 0 ? force_class : pick_tile(dtype, rows, K, N, 256), ga, ea, s);
     };
+    if (dtype != GMLP_F32 && pick_tile(dtype, M, K, N, 256) == TILE_LARGE) {
+      const StreamK sk = plan_streamk(dtype, cdiv(M, 256) * cdiv(K, 256), 2 * (N / 64));
+      if (sk.tiles > 0 && workspace != nullptr && workspace_bytes >= sk.ws_bytes) return run(0, M, false, TILE_LARGE, &sk);
+    }
     int64_t whole = whole_round_tile_rows(dtype, M, K, N);
     if (whole > 0) {
       if (hipError_t err = run(0, whole * 256, false, TILE_LARGE)) return err;
@@ -467,7 +547,7 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
 }
 
 int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_t R, int64_t C,
-                int dtype, void* stream) {
+                int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace gmlp;
   GMLP_REQUIRE_PTR(lhs); GMLP_REQUIRE_PTR(rhs); GMLP_REQUIRE_PTR(dw);
   GMLP_REQUIRE_DTYPE(dtype);
@@ -475,6 +555,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   if (int rc = check_mult8(__func__, "R", R)) return rc;
   if (int rc = check_mult8(__func__, "C", C)) return rc;
   GMLP_REQUIRE_ALIGNED(lhs); GMLP_REQUIRE_ALIGNED(rhs); GMLP_REQUIRE_ALIGNED(dw);
+  GMLP_REQUIRE_ALIGNED(workspace);
 
   // dW[R,C] = lhs[Mred,R]ᵀ · rhs[Mred,C]: both operands reduction-strided.
   GemmArgs ga = {};
@@ -483,6 +564,7 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   ga.M = (int)R; ga.N = (int)C; ga.K = (int)Mred; ga.lda = (int)R; ga.ldb = (int)C;
   ga.nseg = 1; ga.group_m = pick_group(R, C);
   int tc = pick_tile(dtype, R, C, Mred, 256, true);
+  if (tc == TILE_LARGE) use_streamk(plan_streamk(dtype, cdiv(R, 256) * cdiv(C, 256), cdiv(Mred, 64)), ga, workspace, workspace_bytes);
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = by_dtype(dtype, [&](auto tag) {
     typedef decltype(tag) T;
@@ -492,8 +574,23 @@ int gmlp_dw_bwd(const void* lhs, const void* rhs, void* dw, int64_t Mred, int64_
   return hip_result(__func__, e);
 }
 
+size_t gmlp_dw_bwd_grouped_workspace_bytes(int count, int64_t Mred, const int64_t* R, const int64_t* C, int dtype) {
+  using namespace gmlp;
+  if (count < 1 || count > GEMM_GROUP_MAX || R == nullptr || C == nullptr || Mred < 1 || dtype == GMLP_F32) return 0;
+  int64_t tiles256 = 0, tiles128 = 0;
+  for (int i = 0; i < count; ++i) {
+    if (R[i] < 1 || C[i] < 1 || pick_tile(dtype, R[i], C[i], Mred, 256, true) == TILE_MEDIUM) return 0;
+    tiles256 += cdiv(R[i], 256) * cdiv(C[i], 256);
+    tiles128 += cdiv(R[i], 128) * cdiv(C[i], 128);
+  }
+  if (group_tile_class(tiles256, tiles128) != TILE_LARGE) return 0;
+  const StreamK sk = plan_streamk(dtype, tiles256, cdiv(Mred, 64));
+  return sk.tiles > cdiv(R[count - 1], 256) * cdiv(C[count - 1], 256) ? 0 : sk.ws_bytes;
+}
+
 int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rhs, void* const* dw,
-                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* stream) {
+                        int64_t Mred, const int64_t* R, const int64_t* C, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream) {
   using namespace gmlp;
   if (count < 1 || count > GEMM_GROUP_MAX)
     return fail(GMLP_EINVAL, "%s: count = %d must be in 1..%d", __func__, count, GEMM_GROUP_MAX);
@@ -513,7 +610,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
   }
   if (!pipelined) {
     for (int i = 0; i < count; ++i)
-      if (int rc = gmlp_dw_bwd(lhs[i], rhs[i], dw[i], Mred, R[i], C[i], dtype, stream)) return rc;
+      if (int rc = gmlp_dw_bwd(lhs[i], rhs[i], dw[i], Mred, R[i], C[i], dtype, workspace, workspace_bytes, stream)) return rc;
     return GMLP_OK;
   }
   int64_t tiles256 = 0, tiles128 = 0;
@@ -537,7 +634,14 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
   // of them: the pointer moves along the rows and the buffer size is trimmed to match.
   int64_t band_rows = 0, band_cols = 0;  // size of the band, in output rows or columns (one is 0)
   const int last = count - 1;
+  // With a long reduction the last round's tiles (the last ones of the last problem) are shared out
+  // by reduction range instead (stream-K), if the last problem has that many tiles.
+  StreamK sk;
   if (group_class == TILE_LARGE) {
+    sk = plan_streamk(dtype, tiles256, cdiv(Mred, 64));
+    if (sk.tiles > cdiv(R[last], 256) * cdiv(C[last], 256) || workspace == nullptr || workspace_bytes < sk.ws_bytes) sk = StreamK{};
+  }
+  if (group_class == TILE_LARGE && sk.tiles == 0) {
     const int64_t cus = num_cu(), rounds = tiles256 / cus, tail = tiles256 % cus;
     const int64_t tr = (R[last] + 255) / 256, tc = (C[last] + 255) / 256;
     // (worth it for a few rounds only: measured -7 % at 2 rounds, -1 % and less from 8 rounds on)
@@ -563,6 +667,7 @@ int gmlp_dw_bwd_grouped(int count, const void* const* lhs, const void* const* rh
       }
       grp.ga[last].M -= (int)band_rows;
       grp.ga[last].N -= (int)band_cols;
+      use_streamk(sk, grp.ga[last], workspace, workspace_bytes);
       if (hipError_t err = launch_dw_group<T>(group_class, grp, s)) return err;
       if (band_rows == 0 && band_cols == 0) return hipSuccess;
       GemmArgs ga;

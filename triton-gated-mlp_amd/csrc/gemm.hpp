@@ -40,6 +40,16 @@ struct GemmArgs {
                      // for the usual power-of-two row pitches crowds onto a few memory channels.
                      // Workgroups that share B rows keep the same order, so they still share them
                      // in L2.
+  // Stream-K (pipelined kernel, non-split epilogues): the last sk_tiles output tiles (in workgroup
+  // order) are not computed one per workgroup; their reduction tiles are shared out evenly over
+  // sk_wgs extra workgroups at the end of the grid, which leave partial sums in sk_ws
+  // ((sk_wgs + sk_tiles) slots of one output tile's accumulators, fp32), added up in a fixed order
+  // by a second launch.  sk_tiles == 0: every tile has a workgroup of its own.
+  int sk_tiles, sk_wgs;
+  int sk_chunks;     // > 0: sk_wgs == sk_chunks * sk_tiles and every tile is cut into sk_chunks equal
+                     // reduction ranges, one workgroup each (slot = workgroup); 0: even ranges over the
+                     // (tile, reduction tile) sequence, which may straddle tiles
+  float* sk_ws;
   int nxcd;          // accelerator dies of the device (each with its own L2) the hardware deals
                      // workgroup ids to, round-robin (0 is read as 1: no remapping)
 };

@@ -84,7 +84,7 @@ struct PipeConfig {
 };
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
-          typename Epi>
+          typename Epi, bool SK = false>
 __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const typename Epi::Args& ea_in,
                                                     int pid, int nwg) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
@@ -114,37 +114,46 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   const int wm = wave / WGN, wn = wave % WGN;
 
   const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
-  // Workgroup -> (split, tile): all tiles of split 0, then all tiles of split 1, ...
   const int ntiles = tiles_m * tiles_n;
-  const int u = xcd_contiguous(pid, nwg, ga.nxcd);
-  const int split = Epi::SPLIT ? u / ntiles : 0;
-  int tm_i, tn_i;
-  tile_of_grouped(u - split * ntiles, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
-  // workgroup-uniform by construction; say so, the tile origins feed scalar operands
-  const int m0 = __builtin_amdgcn_readfirstlane(tm_i) * BM, n0 = __builtin_amdgcn_readfirstlane(tn_i) * BN;
+  const int kt_seg = (ga.K + BK - 1) / BK;
+  const int kt_all = kt_seg * ga.nseg;  // 64-wide reduction tiles of one output tile
   typename Epi::Args ea = ea_in;
+
+  // What this workgroup computes, as a sequence of pieces (output tile, range of reduction tiles):
+  //   * one whole tile (the usual case; workgroup -> tile in XCD-contiguous, grouped order);
+  //   * with a split-reduction epilogue, one tile's share `split` of the reduction: all tiles of
+  //     split 0, then all tiles of split 1, ...;
+  //   * stream-K (SK, a kernel instance and a launch of its own behind the launch that covers the
+  //     other tiles): ga.sk_wgs workgroups share out the reduction tiles of the problem's last
+  //     ga.sk_tiles output tiles evenly, as one range of (tile, reduction tile) pairs each; a range
+  //     covers the end of one tile and the start of the next (or more), and every piece leaves
+  //     its partial sums in accumulator layout in slot (workgroup + tile) of ga.sk_ws, from where
+  //     streamk_fixup_kernel adds a tile's pieces up in reduction order and runs the epilogue.
+  //     (One kernel with a run-time choice between the epilogue and the partial store was measured
+  //     1.5 to 2 % slower on every launch: the branches sit inside the unrolled epilogue loops, since
+  //     a second loop over the accumulators makes the compiler copy all of them to VGPRs first.)
+  static_assert(!(SK && Epi::SPLIT), "stream-K pieces replace the epilogue");
+  const int dp_tiles = ntiles - (Epi::SPLIT ? 0 : ga.sk_tiles);
+  constexpr bool streamk = SK;
+  int sk_wg = 0;
+  long long sk_cursor = 0, sk_end = 0;  // position in the stream-K iteration space: tile * kt_all + reduction tile
+  if (streamk) {
+    sk_wg = xcd_contiguous(pid, ga.sk_wgs, ga.nxcd);
+    const long long iters = (long long)ga.sk_tiles * kt_all;
+    sk_cursor = iters * sk_wg / ga.sk_wgs;
+    sk_end = iters * (sk_wg + 1) / ga.sk_wgs;
+  }
+  const int u_dp = streamk ? 0 : xcd_contiguous(pid, Epi::SPLIT ? nwg : dp_tiles, ga.nxcd);
+  const int split = Epi::SPLIT ? u_dp / ntiles : 0;
   if constexpr (Epi::SPLIT) ea.ws += (size_t)split * ea.split_stride;
 
-  acc_t acc[G][TM];
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int r = 0; r < (int)(sizeof(acc_t) / 4); ++r) acc[g][i][r] = 0.f;
+  // Per piece (set at the top of the piece loop further down): tile origin, reduction range, the
+  // order in which the range is read from memory (the sum does not mind: see GemmArgs::rotate).
+  int m0 = 0, n0 = 0, kt_first = 0, kt_total = 0, kt_len = 0, rot = 0;
+  uint32_t a_org = 0, b_org = 0;
+  float* partial_slot = nullptr;  // stream-K piece: where its partial sums go
 
-  // This workgroup reduces the 64-wide reduction tiles [kt_first, kt_total) of the concatenated
-  // segments: everything, or its share of a split reduction.
-  const int kt_seg = (ga.K + BK - 1) / BK;
-  int kt_first = 0, kt_total = kt_seg * ga.nseg;
-  if constexpr (Epi::SPLIT) {
-    const int per = (kt_total + ga.splits - 1) / ga.splits;
-    kt_first = split * per;
-    kt_total = kt_first + per < kt_total ? kt_first + per : kt_total;
-  }
-  // Order in which the range is read from memory (the sum does not mind): see GemmArgs::rotate.
-  const int kt_len = kt_total - kt_first;
-  const int rot = ga.rotate && kt_len > 0 ? tn_i % kt_len : 0;
+  acc_t acc[G][TM];
 
   // Per-lane load offsets (constant), per-operand tile origins and per-tile strides (uniform).
   // Buffer addressing uses 32-bit byte offsets from each operand's base; the host checks sizes.
@@ -161,8 +170,6 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
     boff[i] = BTile::lane_offset(i, ga.ldb, wave, lane) + DMA_BIAS - (i & 3) * 1024;
   const uint32_t a_step = A_KS ? (uint32_t)BK * ga.lda * 2 : (uint32_t)BK * 2;
   const uint32_t b_step = B_KS ? (uint32_t)BK * ga.ldb * 2 : (uint32_t)BK * 2;
-  const uint32_t a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
-  const uint32_t b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)smem;
   const uint32_t a_bytes = (uint32_t)(A_KS ? ga.K : ga.M) * ga.lda * 2 + DMA_BIAS - (uint32_t)ga.a_trim;
   const uint32_t b_bytes = (uint32_t)(B_KS ? ga.K : ga.N) * ga.ldb * 2 + DMA_BIAS - (uint32_t)ga.b_trim;
@@ -285,6 +292,56 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
     }
   };
 
+  for (;;) {  // pieces of this workgroup (one, unless stream-K)
+  int u_tile;
+  if (streamk && ga.sk_chunks > 0) {
+    // Whole-number pieces per tile: workgroup w takes reduction chunk w / sk_tiles of tile
+    // w % sk_tiles, so that the workgroups of an XCD (consecutive w) walk neighbouring tiles over the
+    // same reduction range and share operand panels in L2 as the one-tile-per-workgroup grid does.
+    const int s_tile = sk_wg % ga.sk_tiles, chunk = sk_wg / ga.sk_tiles;
+    kt_first = chunk * kt_all / ga.sk_chunks;
+    kt_total = (chunk + 1) * kt_all / ga.sk_chunks;
+    sk_cursor = sk_end = 0;
+    u_tile = dp_tiles + s_tile;
+    partial_slot = ga.sk_ws + (size_t)sk_wg * (size_t)(BM * BN * NB);
+  } else if (streamk) {
+    const unsigned s_tile = (unsigned)sk_cursor / (unsigned)kt_all;
+    const unsigned tile_begin = s_tile * (unsigned)kt_all, tile_end = tile_begin + (unsigned)kt_all;
+    kt_first = (int)((unsigned)sk_cursor - tile_begin);
+    kt_total = (int)(((unsigned)sk_end < tile_end ? (unsigned)sk_end : tile_end) - tile_begin);
+    sk_cursor = tile_begin + (unsigned)kt_total;
+    u_tile = dp_tiles + (int)s_tile;
+    partial_slot = ga.sk_ws + (size_t)(sk_wg + (int)s_tile) * (size_t)(BM * BN * NB);
+  } else {
+    u_tile = u_dp - split * ntiles;
+    kt_first = 0;
+    kt_total = kt_all;
+    if constexpr (Epi::SPLIT) {
+      const int per = (kt_all + ga.splits - 1) / ga.splits;
+      kt_first = split * per;
+      kt_total = kt_first + per < kt_all ? kt_first + per : kt_all;
+    }
+  }
+  {
+    int tm_i, tn_i;
+    tile_of_grouped(u_tile, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+    // workgroup-uniform by construction; say so, the tile origins feed scalar operands
+    m0 = __builtin_amdgcn_readfirstlane(tm_i) * BM;
+    n0 = __builtin_amdgcn_readfirstlane(tn_i) * BN;
+    kt_first = __builtin_amdgcn_readfirstlane(kt_first);
+    kt_total = __builtin_amdgcn_readfirstlane(kt_total);
+    kt_len = kt_total - kt_first;
+    rot = ga.rotate && kt_len > 0 ? tn_i % kt_len : 0;
+    a_org = A_KS ? (uint32_t)m0 * 2 : (uint32_t)m0 * ga.lda * 2;
+    b_org = B_KS ? (uint32_t)n0 * 2 : (uint32_t)n0 * ga.ldb * 2;
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < (int)(sizeof(acc_t) / 4); ++r) acc[g][i][r] = 0.f;
+
   // Prologue: tile 0 .. NS-2 entirely, and of tile NS-1 the loads the handover groups would have
   // issued (tile 0's own slots issue the rest); wait for tile 0.
   constexpr int HEAD_LOADS = (HEAD_SLOTS - LOAD_PHASE + LOAD_SLOTS - 1) / LOAD_SLOTS;
@@ -332,26 +389,37 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // (the operand fragments are still live during the last reduction tile: the first PD_EARLY
   // items are fetched before it, the rest of the PD behind it)
   constexpr int PD_EARLY = PD < 8 ? PD : 8;
+  if (PD > 0 && !streamk) {
 #pragma unroll
-  for (int q = 0; q < PD_EARLY; ++q) {
-    int row, m, n, cg;
-    item_pos(q, row, m, n, cg);
-    Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
+    for (int q = 0; q < PD_EARLY; ++q) {
+      int row, m, n, cg;
+      item_pos(q, row, m, n, cg);
+      Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
+    }
   }
   tile_body(kt, std::false_type{});
+  if (PD > PD_EARLY && !streamk) {
 #pragma unroll
-  for (int q = PD_EARLY; q < PD; ++q) {
-    int row, m, n, cg;
-    item_pos(q, row, m, n, cg);
-    Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
+    for (int q = PD_EARLY; q < PD; ++q) {
+      int row, m, n, cg;
+      item_pos(q, row, m, n, cg);
+      Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
+    }
+    wait_vmem<2 * (PD - PD_EARLY)>();
+  } else {
+    wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
   }
-  if constexpr (PD == PD_EARLY) wait_vmem<0>();  // redundant tail loads must not land in the epilogue's staging area
-  else wait_vmem<2 * (PD - PD_EARLY)>();
 
   // ---- epilogue: transpose MI-row slabs through LDS, after which each lane owns 8 consecutive
   // columns of one row: the fp32 accumulators themselves, with the arithmetic behind the transpose
   // (slabs), or, where the epilogue offers it, the finished 16-bit results (further down).
   __syncthreads();  // all wavefronts are done reading operand tiles
+  // A stream-K piece stores its accumulators as they are instead (16 bytes per lane and
+  // accumulator, contiguous over the wavefront; streamk_fixup_kernel knows the layout).  That
+  // store sits inside the loops below, next to the staging store it replaces: a second loop over
+  // the accumulators in a branch of its own makes the compiler copy all of them to VGPRs first.
+  constexpr int AV = (int)(sizeof(acc_t) / 4);
+  float* const sk_slot = partial_slot + ((size_t)wave * (G * TM) * 64 + lane) * AV;
   constexpr int ELD = Cfg::EPI_LD;
   float* stg = (float*)(smem + wave * Cfg::EPI_WAVE_BYTES);
   const int mrow = lane & (MI - 1), nsub = 4 * (lane / MI);
@@ -371,9 +439,11 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           f32x4 o;
 #pragma unroll
           for (int r = 0; r < 4; ++r) o[r] = acc[g][i][4 * v + r];
-          *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
+          if (streamk) *(f32x4*)(sk_slot + (size_t)(g * TM + i) * 64 * AV + 4 * v) = o;
+          else *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
         }
       }
+      if (streamk) continue;
       // Same-wavefront LDS writes and reads are ordered; no barrier needed for a private slab.
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
@@ -444,6 +514,11 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           if constexpr (NB == 2) v1[r] = acc[TN + j][i][r];
           else v1[r] = 0.f;
         }
+        if (streamk) {
+          *(f32x4*)(sk_slot + (size_t)(j * TM + i) * 64 * AV) = f32x4{v0[0], v0[1], v0[2], v0[3]};
+          if constexpr (NB == 2) *(f32x4*)(sk_slot + (size_t)((TN + j) * TM + i) * 64 * AV) = f32x4{v1[0], v1[1], v1[2], v1[3]};
+          continue;
+        }
         vec4 o[P];
         Epi::pack4(ea, m, n, bias[j], v0, v1, o);
         const int unit = (4 * j + cq) ^ (2 * (mrow >> SH));
@@ -454,6 +529,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
             *(vec4*)(stp + pl * (MI * WTN * 2) + mrow * (WTN * 2) + unit * 8) = o[pl];
         }
       }
+      if (streamk) continue;
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
         int row, m2, n2, cg;
@@ -472,9 +548,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
         }
       }
     }
-    return;
-  }
-  if constexpr (Epi::HAS_ACT) {
+  } else if constexpr (Epi::HAS_ACT) {
     switch (ea.act) {
       case ACT_SILU: slabs(std::integral_constant<int, ACT_SILU>{}); break;
       case ACT_GELU: slabs(std::integral_constant<int, ACT_GELU>{}); break;
@@ -487,13 +561,96 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   } else {
     slabs(std::integral_constant<int, ACT_RUNTIME>{});
   }
+  if (!streamk || (unsigned)sk_cursor >= (unsigned)sk_end) break;
+  __syncthreads();  // the next piece's loads overwrite what this piece's wavefronts were reading
+  }  // pieces
+}
+
+// Second stage of stream-K: adds up the pieces of each stream-K tile in reduction order (fixed, so
+// the result does not depend on timing) and runs the GEMM's epilogue on the sums, four consecutive
+// columns of one row per lane as the accumulators hold them.  Same thread -> element map as
+// gemm_pipelined_body; workgroup (tile, i) handles the MI-row slab i of every wavefront's part of
+// the tile, all its column blocks in flight at once (the kernel is bound by load latency).
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, int NB, typename Epi>
+__global__ void __launch_bounds__(WGM* WGN * 64) streamk_fixup_kernel(GemmArgs ga, typename Epi::Args ea) {
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, false, false, NB> Cfg;
+  static_assert(MI == 16, "accumulator layout of the 16x16x32 MFMA");
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, G = Cfg::G, WTM = Cfg::WTM, WTN = Cfg::WTN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int tiles_m = (ga.M + BM - 1) / BM, tiles_n = (ga.N + BN - 1) / BN;
+  const int dp_tiles = tiles_m * tiles_n - ga.sk_tiles;
+  const int s_tile = blockIdx.x / TM, i = blockIdx.x % TM;
+  int tm_i, tn_i;
+  tile_of_grouped(dp_tiles + s_tile, tiles_m, tiles_n, ga.group_m, tm_i, tn_i);
+  const int m0 = tm_i * BM, n0 = tn_i * BN;
+  const unsigned kt_all = (unsigned)(((ga.K + 63) / 64) * ga.nseg);
+  const unsigned iters = (unsigned)ga.sk_tiles * kt_all, wgs = (unsigned)ga.sk_wgs;
+  const unsigned lo = (unsigned)s_tile * kt_all, hi = lo + kt_all;
+  // first workgroup whose range [iters*w/wgs, iters*(w+1)/wgs) reaches into this tile
+  unsigned w_first = (unsigned)((unsigned long long)lo * wgs / iters);
+  while (w_first > 0 && (unsigned)((unsigned long long)iters * w_first / wgs) > lo) --w_first;
+  while ((unsigned)((unsigned long long)iters * (w_first + 1) / wgs) <= lo) ++w_first;
+  const size_t slot_floats = (size_t)BM * BN * NB;
+  const int mrow = lane & 15, cq = lane >> 4;
+  f32x4 v[NB][TN];
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) v[b][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // the tile's pieces in reduction order: chunk c in slot c * sk_tiles + tile, or the workgroups
+  // whose ranges reach into the tile, workgroup w's piece in slot w + tile
+  const bool chunked = ga.sk_chunks > 0;
+  const unsigned w_begin = chunked ? 0u : w_first;
+  for (unsigned w = w_begin; chunked ? w < (unsigned)ga.sk_chunks
+                                     : (w < wgs && (unsigned)((unsigned long long)iters * w / wgs) < hi); ++w) {
+    const size_t slot_index = chunked ? (size_t)w * ga.sk_tiles + s_tile : (size_t)w + s_tile;
+    const float* slot = ga.sk_ws + slot_index * slot_floats + ((size_t)wave * (G * TM) * 64 + lane) * 4;
+    f32x4 t[NB][TN];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) t[b][j] = *(const f32x4*)(slot + (size_t)((b * TN + j) * TM + i) * 256);
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) v[b][j] += t[b][j];
+  }
+  const int m = m0 + wm * WTM + i * MI + mrow;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * WTN + j * MI + 4 * cq;
+    if (m < ga.M && n < ga.N) {
+      float a0[4] = {v[0][j][0], v[0][j][1], v[0][j][2], v[0][j][3]};
+      float a1[4] = {v[NB - 1][j][0], v[NB - 1][j][1], v[NB - 1][j][2], v[NB - 1][j][3]};
+      Epi::template apply<4>(ea, m, n, a0, a1);
+    }
+  }
 }
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
-          typename Epi>
+          typename Epi, bool SK = false>
 __global__ void __launch_bounds__(WGM* WGN * 64)
     gemm_kernel_pipelined(GemmArgs ga, typename Epi::Args ea) {
-  gemm_pipelined_body<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(ga, ea, blockIdx.x, gridDim.x);
+  gemm_pipelined_body<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi, SK>(ga, ea, blockIdx.x, gridDim.x);
+}
+
+// The stream-K launches behind a launch that left ga.sk_tiles tiles out: the pieces, then the sums.
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
+          typename Epi>
+hipError_t launch_streamk_tail(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
+  if constexpr (!Epi::SPLIT && MI == 16 && BM == 256) {
+    typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+    constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi, true>;
+    if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
+    hipLaunchKernelGGL(kern, dim3(ga.sk_wgs), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, ga, ea);
+    if (hipError_t e = hipGetLastError()) return e;
+    hipLaunchKernelGGL((streamk_fixup_kernel<T, BM, BN, MI, WGM, WGN, NB, Epi>), dim3(ga.sk_tiles * Cfg::TM),
+                       dim3(Cfg::NW * 64), 0, s, ga, ea);
+    return hipGetLastError();
+  } else {
+    return hipErrorInvalidValue;  // the host plans stream-K for the large tiles only
+  }
 }
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
@@ -520,9 +677,14 @@ hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& e
   constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
   if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   const int splits = Epi::SPLIT ? ga.splits : 1;
-  dim3 grid(((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN) * splits), block(Cfg::NW * 64);
-  hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
-  return hipGetLastError();
+  const int tiles = ((ga.M + BM - 1) / BM) * ((ga.N + BN - 1) / BN);
+  const bool sk = !Epi::SPLIT && ga.sk_tiles > 0;
+  dim3 grid(sk ? tiles - ga.sk_tiles : tiles * splits), block(Cfg::NW * 64);
+  if (grid.x > 0) {
+    hipLaunchKernelGGL(kern, grid, block, Cfg::LDS_BYTES, s, ga, ea);
+    if (hipError_t e = hipGetLastError()) return e;
+  }
+  return sk ? launch_streamk_tail<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(ga, ea, s) : hipSuccess;
 }
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
@@ -534,11 +696,17 @@ hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipSt
   int total = 0;
   for (int g = 0; g < grp.count; ++g) {
     grp.first[g] = total;
-    total += ((grp.ga[g].M + BM - 1) / BM) * ((grp.ga[g].N + BN - 1) / BN);
+    const int tiles = ((grp.ga[g].M + BM - 1) / BM) * ((grp.ga[g].N + BN - 1) / BN);
+    total += tiles - grp.ga[g].sk_tiles;
   }
   for (int g = grp.count; g <= GEMM_GROUP_MAX; ++g) grp.first[g] = total;
   hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);
-  return hipGetLastError();
+  if (hipError_t e = hipGetLastError()) return e;
+  for (int g = 0; g < grp.count; ++g) {
+    if (grp.ga[g].sk_tiles <= 0) continue;
+    if (hipError_t e = launch_streamk_tail<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(grp.ga[g], grp.ea[g], s)) return e;
+  }
+  return hipSuccess;
 }
 
 }  // namespace gmlp

@@ -16,6 +16,7 @@ from torch import Tensor
 
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD, GMLP_OP_GATEUP_FWD = 0, 1, 2, 3, 4
+GMLP_OP_DH_BWD, GMLP_OP_DW_BWD, GMLP_OP_DW_BWD_GROUPED = 5, 6, 7
 ABI_VERSION = 7
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
@@ -49,11 +50,18 @@ _SIGNATURES = {
         [_c_ptr] * 9 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr, ctypes.c_size_t, _c_ptr],
     ),
     "gmlp_linear_fwd": (_int, [_c_ptr] * 4 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
-    "gmlp_dh_bwd": (_int, [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_dh_bwd": (
+        _int,
+        [_c_ptr] * 6 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr, ctypes.c_size_t, _c_ptr],
+    ),
     "gmlp_gating_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr]),
     "gmlp_dx_bwd": (_int, [_c_ptr] * 5 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
-    "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr]),
-    "gmlp_dw_bwd_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _c_ptr, _int, _c_ptr]),
+    "gmlp_dw_bwd": (_int, [_c_ptr] * 3 + [_i64, _i64, _i64, _int, _c_ptr, ctypes.c_size_t, _c_ptr]),
+    "gmlp_dw_bwd_grouped_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _c_ptr, _c_ptr, _int]),
+    "gmlp_dw_bwd_grouped": (
+        _int,
+        [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _c_ptr, _int, _c_ptr, ctypes.c_size_t, _c_ptr],
+    ),
     "gmlp_colsum": (_int, [_c_ptr] * 3 + [_i64, _i64, _int, _c_ptr]),
     "gmlp_colsum_static": (_int, [_c_ptr] * 2 + [_i64, _i64, _int, _c_ptr]),
     "gmlp_colsum_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _int, _c_ptr]),

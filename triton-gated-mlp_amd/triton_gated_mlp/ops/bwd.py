@@ -40,10 +40,12 @@ def dh_bwd(
     du = torch.empty_like(u)
     if M > 0:
         with torch.cuda.device(dev):
+            ws = _cabi.workspace(_cabi.GMLP_OP_DH_BWD, M, K, N, code, dev)
             _cabi.check(
                 _cabi.lib().gmlp_dh_bwd(
                     _cabi.ptr(dy), _cabi.ptr(W_down), _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(dg), _cabi.ptr(du),
-                    M, K, N, code, act, float(dropout_p), int(seed), int(offset), _cabi.stream_ptr(dev),
+                    M, K, N, code, act, float(dropout_p), int(seed), int(offset),
+                    _cabi.ptr(ws), 0 if ws is None else ws.numel(), _cabi.stream_ptr(dev),
                 )
             )
     return dg, du
@@ -114,9 +116,11 @@ def dw_bwd(lhs: Tensor, rhs: Tensor) -> Tensor:
         return torch.zeros((R, C), dtype=lhs.dtype, device=dev)
     dw = torch.empty((R, C), dtype=lhs.dtype, device=dev)
     with torch.cuda.device(dev):
+        ws = _cabi.workspace(_cabi.GMLP_OP_DW_BWD, M, R, C, code, dev)
         _cabi.check(
             _cabi.lib().gmlp_dw_bwd(
-                _cabi.ptr(lhs), _cabi.ptr(rhs), _cabi.ptr(dw), M, R, C, code, _cabi.stream_ptr(dev)
+                _cabi.ptr(lhs), _cabi.ptr(rhs), _cabi.ptr(dw), M, R, C, code,
+                _cabi.ptr(ws), 0 if ws is None else ws.numel(), _cabi.stream_ptr(dev),
             )
         )
     return dw
@@ -147,11 +151,16 @@ def dw_bwd_grouped(pairs):
     R = I64Arr(*[a.shape[1] for a, _ in pairs])
     C = I64Arr(*[b.shape[1] for _, b in pairs])
     with torch.cuda.device(dev):
+        nbytes = _cabi.lib().gmlp_dw_bwd_grouped_workspace_bytes(
+            n, M, ctypes.cast(R, ctypes.c_void_p), ctypes.cast(C, ctypes.c_void_p), code
+        )
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
         _cabi.check(
             _cabi.lib().gmlp_dw_bwd_grouped(
                 n, ctypes.cast(lhs, ctypes.c_void_p), ctypes.cast(rhs, ctypes.c_void_p),
                 ctypes.cast(dws, ctypes.c_void_p), M, ctypes.cast(R, ctypes.c_void_p),
-                ctypes.cast(C, ctypes.c_void_p), code, _cabi.stream_ptr(dev),
+                ctypes.cast(C, ctypes.c_void_p), code, _cabi.ptr(ws), 0 if ws is None else ws.numel(),
+                _cabi.stream_ptr(dev),
             )
         )
     return outs
