@@ -519,7 +519,9 @@ int gmlp_dx_bwd(const void* dg, const void* du, const void* w_gate, const void* 
       if (sk) use_streamk(*sk, ga, workspace, workspace_bytes);
       ga.A[0] = (const T*)dg + row0 * N; ga.A[1] = (const T*)du + row0 * N; ga.B[0] = w_gate; ga.B[1] = w_up;
       ga.M = (int)rows; ga.N = (int)K; ga.K = (int)N; ga.lda = (int)N; ga.ldb = (int)K;
-      ga.nseg = 2; ga.group_m = pick_group(rows, K); ga.rotate = rows <= 512;
+      ga.nseg = 2; ga.group_m = pick_group(rows, K);
+      // (no rotated reduction order here: a piece has room for one change of direction, and with
+      // two reduction segments that is the step from dG·W_gate to dU·W_up)
       typename EpiStore<T>::Args ea = {(T*)dx + row0 * K, nullptr, (int)K};
       if constexpr (!std::is_same<T, float>::value) {
         const int splits = may_split ? pick_splits(dtype, rows, K, N, 2 * ((N + 63) / 64)) : 1;

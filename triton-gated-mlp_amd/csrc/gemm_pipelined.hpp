@@ -104,6 +104,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // keep away from them.
   constexpr int LOAD_PHASE = LOAD_SLOTS >= 4 ? 2 : 0;
   static_assert(LOAD_SLOTS >= 1 && L * LOAD_SLOTS <= TILE_SLOTS, "a tile's loads must fit a tile");
+  static_assert((L - 1) * LOAD_SLOTS + LOAD_PHASE < HEAD_SLOTS + (KSTEPS - 1) * G * TM + TM - 1,
+                "a tile's last load goes out before the load state moves on (first group of the last step)");
 
   extern __shared__ __align__(1024) char smem_raw[];
   char* smem = smem_raw;
@@ -195,26 +197,73 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
       set_lds_dma_base(s + ATile::BYTES + bsel * BTile::BYTES + (wave * BTile::PER_WAVE + i) * 1024);
     }
   };
-  // The load itself (M0 must hold its group's base).  Tiles past the end are replaced by the last
-  // tile: the ring then always holds a full tile in flight, the redundant copies land in slots
-  // nobody reads again.
-  auto issue_one = [&](int kt_req, int x) __attribute__((always_inline)) {
-    int kt = kt_req < kt_total ? kt_req : kt_total - 1;
-    kt += rot;
-    kt = kt >= kt_total ? kt - kt_len : kt;
-    int seg = kt >= kt_seg ? 1 : 0;
-    int kk = kt - seg * kt_seg;
+  // Where the loads of ONE reduction tile read from, as scalar state that moves on tile by tile
+  // through the piece's tiles in the order they are read.  Moving on is two scalar additions, and
+  // at most once per piece something else: the step into the second reduction segment (other
+  // operands: dX only) or the wrap-around of a rotated range (see rot; the host never asks for
+  // both).  That event is prepared when the piece starts and applied without a branch: a branch
+  // inside the unrolled tile body makes the register allocator shuffle accumulators, and
+  // recomputing the addresses per load, as the kernel first did, cost some 35 scalar instructions
+  // per tile in two clumps, each of which held up the MFMA issue for a dozen slots.  Beyond the
+  // piece's last tile the state simply keeps stepping: only the few loads that the last but one
+  // tile issues ahead read there, into a ring slot nobody reads again, and whatever lies beyond
+  // the end of an operand reads as zeros.
+  uint32_t ld_soff_a = 0, ld_soff_b = 0, ld_event_a = 0, ld_event_b = 0;
+  // (the two segments' descriptors differ in their first two words only, the base address: the
+  // state keeps those as one 64-bit scalar per operand, so that switching is one select each)
+  auto rsrc_head = [](const buffer_rsrc& r) __attribute__((always_inline)) {
+    return (uint64_t)(uint32_t)r[0] | ((uint64_t)(uint32_t)r[1] << 32);
+  };
+  uint64_t ld_head_a = rsrc_head(ra[0]), ld_head_b = rsrc_head(rb[0]);
+  int ld_countdown = -1;  // advances left before the event; negative: none to come
+  bool ld_event_seg = false;
+  auto load_state_start = [&]() __attribute__((always_inline)) {
+    int kt = kt_first + rot;
+    const int seg = kt >= kt_seg ? 1 : 0;
+    const int kk = kt - seg * kt_seg;
+    ld_soff_a = a_org + kk * a_step;
+    ld_soff_b = b_org + kk * b_step;
+    ld_head_a = rsrc_head(seg ? ra[1] : ra[0]);
+    ld_head_b = rsrc_head(seg ? rb[1] : rb[0]);
+    ld_countdown = -1;
+    ld_event_seg = false;
+    if (rot > 0) {  // wrap around from the range's last tile to its first
+      const int seg0 = kt_first >= kt_seg ? 1 : 0, kk0 = kt_first - seg0 * kt_seg;
+      ld_countdown = kt_total - 1 - kt;
+      ld_event_a = a_org + kk0 * a_step;
+      ld_event_b = b_org + kk0 * b_step;
+    } else if (seg == 0 && kt_total > kt_seg) {  // on into the second segment
+      ld_countdown = kt_seg - 1 - kk;
+      ld_event_a = a_org;
+      ld_event_b = b_org;
+      ld_event_seg = true;
+    }
+  };
+  auto load_state_advance = [&]() __attribute__((always_inline)) {
+    const bool fire = ld_countdown == 0;
+    const uint32_t na = ld_soff_a + a_step, nb = ld_soff_b + b_step;
+    ld_soff_a = fire ? ld_event_a : na;
+    ld_soff_b = fire ? ld_event_b : nb;
+    ld_countdown -= 1;
+    if constexpr (NB == 1) {  // (two accumulator sets: one reduction segment by construction)
+      const bool sw = fire && ld_event_seg;
+      ld_head_a = sw ? rsrc_head(ra[1]) : ld_head_a;
+      ld_head_b = sw ? rsrc_head(rb[1]) : ld_head_b;
+    }
+  };
+  // Load x of the tile the state stands at (M0 must hold its group's base).
+  auto issue_one = [&](int x) __attribute__((always_inline)) {
     buffer_rsrc r;
     uint32_t voff, soff;
     if (x < ATile::PER_WAVE) {
-      r = seg ? ra[1] : ra[0];
+      r = buffer_rsrc{(int)(uint32_t)ld_head_a, (int)(uint32_t)(ld_head_a >> 32), ra[0][2], ra[0][3]};
       voff = aoff[x];
-      soff = a_org + kk * a_step;
+      soff = ld_soff_a;
     } else {
       int y = x - ATile::PER_WAVE, bsel = y / BTile::PER_WAVE, i = y % BTile::PER_WAVE;
-      r = NB == 2 ? rb[bsel] : (seg ? rb[1] : rb[0]);
+      r = NB == 2 ? rb[bsel] : buffer_rsrc{(int)(uint32_t)ld_head_b, (int)(uint32_t)(ld_head_b >> 32), rb[0][2], rb[0][3]};
       voff = boff[i];
-      soff = b_org + kk * b_step;
+      soff = ld_soff_b;
     }
     switch (load_index(x) & 3) {
       case 0: load16_to_lds_at<0>(r, voff, soff); break;
@@ -278,11 +327,13 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           // --- paced refill of the ring slot retired at the last barrier; slots are counted from
           // that barrier, so a tile's loads start in the previous tile's handover groups.  Load x
           // goes to slot x*LOAD_SLOTS + LOAD_PHASE, a new M0 one slot earlier.
+          // --- the load state moves on from tile kt+1, whose last load went out during the first
+          // step, to tile kt+2: in a slot of the last step that has nothing else to issue
+          if (NEXT && last && g == 0 && i == TM - 1) load_state_advance();
           if (NEXT) {
             const int slot = handover ? (g - (G - LA)) * TM + i : HEAD_SLOTS + (ks * G + g) * TM + i;
             const int lkt = handover ? kt + NS : kt + NS - 1;
-            if (slot % LOAD_SLOTS == LOAD_PHASE && slot / LOAD_SLOTS < L)
-              issue_one(lkt, slot / LOAD_SLOTS);
+            if (slot % LOAD_SLOTS == LOAD_PHASE && slot / LOAD_SLOTS < L) issue_one(slot / LOAD_SLOTS);
             const int nx = (slot + 1) / LOAD_SLOTS;
             if ((slot + 1) % LOAD_SLOTS == LOAD_PHASE && nx < L && starts_group(nx)) dma_base(lkt, nx);
           }
@@ -346,15 +397,17 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // issued (tile 0's own slots issue the rest); wait for tile 0.
   constexpr int HEAD_LOADS = (HEAD_SLOTS - LOAD_PHASE + LOAD_SLOTS - 1) / LOAD_SLOTS;
   constexpr int L_HEAD = HEAD_LOADS < L ? HEAD_LOADS : L;
+  load_state_start();
 #pragma unroll
   for (int x = 0; x < L; ++x) {
     if (starts_group(x)) dma_base(kt_first, x);
-    issue_one(kt_first, x);
+    issue_one(x);
   }
+  load_state_advance();
 #pragma unroll
   for (int x = 0; x < L_HEAD; ++x) {
     if (starts_group(x)) dma_base(kt_first + 1, x);
-    issue_one(kt_first + 1, x);
+    issue_one(x);
   }
   wait_vmem<L_HEAD>();
   __syncthreads();
