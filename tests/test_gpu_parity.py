@@ -120,6 +120,36 @@ def test_cfg3_fp16_forward_backward_llama3_8b():
     _run_module_case(CFG3)
 
 
+def test_cfg3_weight_gradient_tolerance_yardstick():
+    """Why weight gradients are held to atol = 2e-2 * max(1, mean|ref|): an element of dW sums M = 8192
+    products of operands rounded to fp16, so its error has an absolute size set by the typical
+    magnitude of dW (tens), whatever the element's own value; elements much smaller than typical
+    cannot meet a bound relative to themselves.  The yardstick is torch's own fp16 path (hipBLASLt
+    GEMMs on the same rounded dG and x) against the same fp32 oracle: it leaves the plain
+    2e-2/2e-2 band for as many elements as the fused kernels do, and the fused result is as close to
+    the oracle as torch's."""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(3)
+    M, K, N = CFG3.M, CFG3.K, CFG3.N
+    dg = torch.randn(M, N, generator=g).half()
+    x = torch.randn(M, K, generator=g).half()
+    ref = (dg.float().T.to(dev) @ x.float().to(dev)).cpu()  # fp32 products and sums of the rounded operands
+    fused = ops_bwd.dw_bwd(dg.to(dev), x.to(dev)).float().cpu()
+    eager = (dg.to(dev).T @ x.to(dev)).float().cpu()
+    band = ATOL + RTOL * ref.abs()
+    out_fused = int(((fused - ref).abs() > band).sum())
+    out_eager = int(((eager - ref).abs() > band).sum())
+    err_fused, err_eager = (fused - ref).abs().max().item(), (eager - ref).abs().max().item()
+    print(f"  mean|dW|={ref.abs().mean().item():.1f}  outside plain band: fused {out_fused}, torch fp16 {out_eager} of {ref.numel()}; "
+          f"max_abs_err fused {err_fused:.3e}, torch fp16 {err_eager:.3e}", flush=True)
+    assert out_fused <= max(2 * out_eager, 1000)
+    assert err_fused <= 2.0 * err_eager
+    scale = max(1.0, ref.abs().mean().item())
+    assert ((fused - ref).abs() <= ATOL * scale + RTOL * ref.abs()).all()
+
+
 def test_cfg4_bf16_bias_dropout_forward_backward():
     _run_module_case(CFG4)
 
