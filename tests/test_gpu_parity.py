@@ -51,7 +51,7 @@ def _oracle_inputs(t):
     return {k: (None if v is None else v.float()) for k, v in t.items()}
 
 
-def _run_module_case(c: Case, lean: bool = False):
+def _run_module_case(c: Case, lean: bool = False, yardstick: bool = False):
     from triton_gated_mlp import FusedGatedMLP
     from triton_gated_mlp.ops import fwd as ops_fwd
 
@@ -110,6 +110,24 @@ def _run_module_case(c: Case, lean: bool = False):
         # weight gradients sum M terms: scale the absolute tolerance with the magnitude of the result
         scale = max(1.0, ref[n].abs().mean().item())
         _close(n, g, ref[n], atol=ATOL * scale)
+    if yardstick:
+        from triton_gated_mlp import EagerGatedMLP, copy_weights
+
+        eager = EagerGatedMLP(hidden_size=c.K, intermediate_size=c.N, bias=c.bias, dropout_p=0.0, hidden_act=c.act)
+        eager = eager.to(dev).to(c.dtype)
+        copy_weights(mlp, eager)
+        xe = t["x"].to(dev).requires_grad_(True)
+        ge = torch.autograd.grad(eager(xe), [xe, eager.gate_proj.weight, eager.up_proj.weight, eager.down_proj.weight],
+                                 grad_outputs=t["dY"].to(dev))
+        for n, g_fused, g_eager in zip(names[:4], grads[:4], ge):
+            r = ref[n]
+            band = ATOL + RTOL * r.abs()
+            e_f, e_e = (g_fused.float().cpu() - r).abs(), (g_eager.float().cpu() - r).abs()
+            out_f, out_e = int((e_f > band).sum()), int((e_e > band).sum())
+            print(f"  yardstick {n}: outside plain band fused {out_f}, torch fp16 {out_e} of {r.numel()}; "
+                  f"max_abs_err fused {e_f.max().item():.3e}, torch fp16 {e_e.max().item():.3e}", flush=True)
+            assert out_f <= 1.5 * out_e + 1000, f"{n}: the fused path leaves the plain band far more often than torch's fp16 path"
+            assert e_f.max().item() <= 2.0 * e_e.max().item() + ATOL
 
 
 def test_cfg2_fp16_forward_llama7b():
@@ -117,37 +135,14 @@ def test_cfg2_fp16_forward_llama7b():
 
 
 def test_cfg3_fp16_forward_backward_llama3_8b():
-    _run_module_case(CFG3)
-
-
-def test_cfg3_weight_gradient_tolerance_yardstick():
-    """Why weight gradients are held to atol = 2e-2 * max(1, mean|ref|): an element of dW sums M = 8192
-    products of operands rounded to fp16, so its error has an absolute size set by the typical
-    magnitude of dW (tens), whatever the element's own value; elements much smaller than typical
-    cannot meet a bound relative to themselves.  The yardstick is torch's own fp16 path (hipBLASLt
-    GEMMs on the same rounded dG and x) against the same fp32 oracle: it leaves the plain
-    2e-2/2e-2 band for as many elements as the fused kernels do, and the fused result is as close to
-    the oracle as torch's."""
-    from triton_gated_mlp.ops import bwd as ops_bwd
-
-    dev = _dev()
-    g = torch.Generator().manual_seed(3)
-    M, K, N = CFG3.M, CFG3.K, CFG3.N
-    dg = torch.randn(M, N, generator=g).half()
-    x = torch.randn(M, K, generator=g).half()
-    ref = (dg.float().T.to(dev) @ x.float().to(dev)).cpu()  # fp32 products and sums of the rounded operands
-    fused = ops_bwd.dw_bwd(dg.to(dev), x.to(dev)).float().cpu()
-    eager = (dg.to(dev).T @ x.to(dev)).float().cpu()
-    band = ATOL + RTOL * ref.abs()
-    out_fused = int(((fused - ref).abs() > band).sum())
-    out_eager = int(((eager - ref).abs() > band).sum())
-    err_fused, err_eager = (fused - ref).abs().max().item(), (eager - ref).abs().max().item()
-    print(f"  mean|dW|={ref.abs().mean().item():.1f}  outside plain band: fused {out_fused}, torch fp16 {out_eager} of {ref.numel()}; "
-          f"max_abs_err fused {err_fused:.3e}, torch fp16 {err_eager:.3e}", flush=True)
-    assert out_fused <= max(2 * out_eager, 1000)
-    assert err_fused <= 2.0 * err_eager
-    scale = max(1.0, ref.abs().mean().item())
-    assert ((fused - ref).abs() <= ATOL * scale + RTOL * ref.abs()).all()
+    """The headline configuration at full size.  Also the yardstick for the weight-gradient tolerance
+    (atol = 2e-2 * max(1, mean|ref|)): an element of dW sums M = 8192 products of operands that were
+    themselves rounded to fp16 on the way (dG, dU, H), so its error has an absolute size set by the
+    typical magnitude of dW (tens), whatever the element's own value, and elements far below typical
+    cannot meet a bound relative to themselves.  torch's own fp16 module (EagerGatedMLP on the GPU,
+    hipBLASLt GEMMs) is run on the same inputs: against the same fp32 oracle it leaves the plain
+    2e-2/2e-2 band for about as many elements, and the fused gradients are as close as torch's."""
+    _run_module_case(CFG3, yardstick=True)
 
 
 def test_cfg4_bf16_bias_dropout_forward_backward():
