@@ -13,8 +13,9 @@
  *   - dtype: GMLP_F16 or GMLP_BF16 storage (the tuned kernels) or GMLP_F32 (compatibility path on
  *     fp32 MFMA, not tuned; not for gmlp_decode_fwd); accumulation and epilogue arithmetic are fp32.
  *   - Every call only ENQUEUES work on `stream` (a hipStream_t; NULL = default stream) and returns.
- *     The library never allocates, frees or keeps device memory; the caller owns every buffer,
- *     including workspaces (sizes from gmlp_workspace_bytes).
+ *     The library never allocates or frees device memory and keeps no pointer past a call; the
+ *     caller owns every buffer, including workspaces (sizes from gmlp_workspace_bytes).  The one
+ *     piece of device memory of its own is the static scratch array of gmlp_colsum_static.
  *   - Return value: 0 on success, a negative GMLP_E* code otherwise; nothing is launched on error.
  *     gmlp_last_error() returns a thread-local message for the last failing call on this thread.
  *   - Dropout: keep(m,n) = philox4x32_10(counter = {lo32(e/4), hi32(e/4), lo32(offset), hi32(offset)},
