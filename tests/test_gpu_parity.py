@@ -829,6 +829,14 @@ def test_streamk_seams_every_gemm_kind_against_fp32_matmul():
     assert (y.float() - y0.float()).abs().max().item() <= 2e-3 * y0.float().abs().max().item()
     assert not torch.equal(y, torch.zeros_like(y))
 
+    # the same with ragged edges (2000 rows, 11256 columns) in bf16: pieces of edge tiles, predicated sums
+    M, R, C = 2000, 5184, 11256
+    assert _streamk_expected(_cabi.GMLP_OP_LINEAR_FWD, M, R, C, 1) == (96 + 256) * 65536 * 4
+    a, w, b = [v.bfloat16() for v in (rnd(M, R), rnd(C, R, s=0.02), rnd(C, s=0.1))]
+    y = ops_fwd.linear_fwd(a.to(dev), w.to(dev), b.to(dev))
+    assert torch.equal(y, ops_fwd.linear_fwd(a.to(dev), w.to(dev), b.to(dev)))
+    _close("linear stream-K ragged bf16", y, f(a) @ f(w).T + f(b))
+
     # gate/up: [2048, 5120] hidden = 8 x 40 tiles of 256 x 128, reduction 4352; biases, dropout, G and U kept
     M, K, N = 2048, 4352, 5120
     assert _streamk_expected(_cabi.GMLP_OP_GATEUP_FWD, M, K, N) > 0

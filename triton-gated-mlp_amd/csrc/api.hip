@@ -12,6 +12,10 @@
 
 #include "launch.hpp"
 
+#ifndef GMLP_MI
+#define GMLP_MI 16  // MFMA shape of the GEMM units (a build-wide knob: make EXTRA=-DGMLP_MI=32)
+#endif
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -195,6 +199,7 @@ struct StreamK {
 StreamK plan_streamk(int dtype, int64_t tiles, int64_t kt) {
   StreamK p;
   const int64_t cus = num_cu(), tail = tiles % cus;
+  if (GMLP_MI != 16) return p;  // the second stage knows the accumulator layout of the 16x16x32 MFMA only
   if (dtype == GMLP_F32 || tail == 0 || kt < 8) return p;
   if ((double)(cus - tail) / (double)cus * (double)kt <= 50.0) return p;
   int64_t wgs = tail * kt / 8;
