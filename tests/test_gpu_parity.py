@@ -891,6 +891,53 @@ def test_streamk_seams_every_gemm_kind_against_fp32_matmul():
         _close("dW grouped stream-K", got, f(a_).T @ f(b_), atol=ATOL * 40)
 
 
+def test_random_shapes_every_operator_against_fp32_products():
+    """Two dozen seeded random shapes through the five GEMM operators: token counts from 1 to a few
+    thousand, widths that are multiples of 64 (tuned kernels: large, medium, two-launch, split and
+    stream-K grids as the dispatcher picks them) or only of 8 (predicated kernel), both 16-bit
+    dtypes; each result against the fp32 product of the same rounded operands (torch's fp32 matmul
+    on the device), and the gate/up and dH epilogues against the oracle's closed forms."""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    rng = np.random.default_rng(20240611)
+    g = torch.Generator(device="cpu").manual_seed(99)
+    f = lambda t: t.float()
+    for case in range(24):
+        dtype = torch.float16 if case % 2 == 0 else torch.bfloat16
+        unit = 8 if case % 6 == 5 else 64
+        M = int(rng.choice([1, 7, 33, 100, 255, 256, 257, 700, 1500, 2304, 3000]))
+        K = int(rng.integers(1, 3072 // unit + 1)) * unit
+        N = int(rng.integers(1, 4096 // unit + 1)) * unit
+        print(f"random case {case}: M={M} K={K} N={N} {dtype}", flush=True)
+        rnd = lambda *shape, s=1.0: (s * torch.randn(*shape, generator=g)).to(dtype).to(dev)
+        x, wg, wu, wd = rnd(M, K), rnd(N, K, s=0.03), rnd(N, K, s=0.03), rnd(K, N, s=0.03)
+        dy = rnd(M, K)
+        # forward
+        hs = ops_fwd.gateup_fwd(x, wg, None, wu, None, save_activations=True)
+        G, U = f(x) @ f(wg).T, f(x) @ f(wu).T
+        _close("G", hs.gate, G)
+        _close("U", hs.up, U)
+        _close("H", hs.hidden, torch.nn.functional.silu(G) * U)
+        y = ops_fwd.linear_fwd(hs.hidden, wd)
+        _close("Y", y, f(hs.hidden) @ f(wd).T, atol=ATOL * max(1.0, (N / 1024) ** 0.5))
+        # backward, from the device's own (rounded) G, U and H so that every operator is checked alone
+        dg, du = ops_bwd.dh_bwd(dy, wd, hs.gate, hs.up)
+        hb = oracle.hidden_backward((f(dy) @ f(wd)).cpu(), f(hs.gate).cpu(), f(hs.up).cpu(), None, 0.0)
+        scale = max(1.0, (K / 1024) ** 0.5)
+        _close("dG", dg, hb["dG"], atol=ATOL * scale)
+        _close("dU", du, hb["dU"], atol=ATOL * scale)
+        dx = ops_bwd.dx_bwd(dg, du, wg, wu)
+        ref_dx = f(dg) @ f(wg) + f(du) @ f(wu)
+        _close("dX", dx, ref_dx, atol=ATOL * max(1.0, ref_dx.abs().mean().item()))
+        pairs = [(dg, x), (du, x), (dy, hs.hidden)]
+        for name, got, (a_, b_) in zip(("dW_gate", "dW_up", "dW_down"), ops_bwd.dw_bwd_grouped(pairs), pairs):
+            ref = f(a_).T @ f(b_)
+            _close(name, got, ref, atol=ATOL * max(1.0, ref.abs().mean().item(), (M / 64) ** 0.5))
+        _close("dW_gate alone", ops_bwd.dw_bwd(dg, x), f(dg).T @ f(x), atol=ATOL * max(1.0, (M / 64) ** 0.5))
+
+
 def test_grouped_weight_gradients_equal_single_launches():
     """gmlp_dw_bwd_grouped (one grid) is bit-identical to three gmlp_dw_bwd launches."""
     from triton_gated_mlp.ops import bwd as ops_bwd
