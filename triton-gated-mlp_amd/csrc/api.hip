@@ -208,8 +208,8 @@ StreamK plan_streamk(int dtype, int64_t tiles, int64_t kt) {
   p.tiles = (int)tail;
   p.wgs = (int)wgs;
   // A whole number of pieces per tile when that still fills (nearly) all compute units: the
-  // workgroups of an XCD then share operand panels (measured on 128 tiles in halves: the pieces'
-  // launch 123 -> see DESIGN).
+  // workgroups of an XCD then walk neighbouring tiles over the same reduction range and share
+  // operand panels in L2 (measured on 128 tiles in halves: the pieces' launch 123 -> 116 us).
   const int64_t per_tile = wgs / tail;
   if (per_tile >= 2 && per_tile * tail * 10 >= wgs * 9 && kt / per_tile >= 8) {
     p.chunks = (int)per_tile;
