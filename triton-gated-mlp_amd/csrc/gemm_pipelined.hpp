@@ -3,7 +3,8 @@
 // Same contract as gemm_kernel (gemm.hpp): C[M,N] = sum_s sum_k A_s[m,k] * B_s[n,k], operands
 // reduction-contiguous (KC) or reduction-strided (KS), NB accumulator sets, fused epilogue.
 // Reduction tiles of 64 elements travel global -> LDS without passing through registers
-// (gemm_tiles.hpp) into a two-slot ring; the epilogue transposes accumulators (or finished
+// (gemm_tiles.hpp) into a two-slot ring (three slots for the A operand of the plain-store GEMMs with a
+// long reduction, see PipeConfig::A3); the epilogue transposes accumulators (or finished
 // results) through LDS so that every global access is a 16-byte, row-contiguous one.
 //
 // Ragged edges cost nothing in the main loop: operands are read through buffer descriptors of
@@ -59,7 +60,21 @@ __device__ __forceinline__ typename AccType<MI>::type mfma_mi(typename Traits<T>
   else return Traits<T>::mfma16(a, b, c);
 }
 
-template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB>
+// Kernels that get the three-entry A ring (see PipeConfig::A3): those with a reduction-contiguous A
+// operand other than dH, i.e. gate/up, the down projection and the input gradient.  The long
+// reductions over the intermediate size gain most (they stall on a full vector-memory queue
+// otherwise), gate/up gains from a cold start only.  dH's epilogue prefetch and the weight
+// gradients' two transposed operands leave no registers for it (spills when tried).
+template <typename T, typename Epi>
+constexpr bool wants_ring_a3() {
+#ifdef GMLP_NO_RING_A3
+  return false;
+#else
+  return !std::is_same<Epi, EpiDh<T>>::value;
+#endif
+}
+
+template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB, bool RING_A3 = false>
 struct PipeConfig {
   static constexpr int BK = 64, NS = 2;
   static constexpr int NW = WGM * WGN;
@@ -74,7 +89,15 @@ struct PipeConfig {
   static constexpr int LOADS = ATile::PER_WAVE + NB * BTile::PER_WAVE;  // per wave per tile
   static constexpr int EPI_LD = WTN + 4;                                // fp32 staging row
   static constexpr int EPI_WAVE_BYTES = NB * MI * EPI_LD * 4;
-  static constexpr int MAIN_BYTES = NS * STAGE;
+  // A3: THREE ring entries of the A operand and two of the B operand(s), all of a workgroup's
+  // 160 KiB.  The A loads of a tile then have two tiles' time to land, so a tile's loads can be
+  // spread evenly over the tile (B in its first half, A in its second) instead of going out back
+  // to back at the rate the texture addresser can take at best, which is where a load that misses
+  // L2 backs the queue up into the issuing wavefronts (down projection: queue-full stalls 166 -> 10
+  // clocks per tile, 2664 -> 2451 clocks per tile, -4 % run time; input gradient -2 %).
+  static constexpr bool A3 = RING_A3 && BM == 256 && MI == 16 && !A_KS;
+  static constexpr int MAIN_BYTES = A3 ? 3 * ATile::BYTES + NS * NB * BTile::BYTES : NS * STAGE;
+  static_assert(MAIN_BYTES <= 160 * 1024, "a workgroup has 160 KiB of LDS");
   static constexpr int LDS_BYTES = MAIN_BYTES > NW * EPI_WAVE_BYTES ? MAIN_BYTES : NW * EPI_WAVE_BYTES;
   static_assert(G >= 2 && TM >= 2 && TM % 2 == 0, "rolling scheme needs >= 2 groups and an even TM");
   static_assert((KSTEPS * G) % 4 == 0, "B ring index must be static");
@@ -87,7 +110,7 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
           typename Epi, bool SK = false>
 __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const typename Epi::Args& ea_in,
                                                     int pid, int nwg) {
-  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, wants_ring_a3<T, Epi>()> Cfg;
   typedef typename Cfg::ATile ATile;
   typedef typename Cfg::BTile BTile;
   typedef typename Traits<T>::vec8 vec8;
@@ -97,6 +120,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   constexpr int KSTEPS = Cfg::KSTEPS, STAGE = Cfg::STAGE, L = Cfg::LOADS;
   constexpr int LOAD_SLOTS = GMLP_LOAD_CYCLES / Cfg::MFMA_CYCLES;  // MFMA slots per load
   constexpr int TILE_SLOTS = KSTEPS * G * TM;                         // MFMA slots per tile
+  constexpr bool A3 = Cfg::A3;
   constexpr int LA = GMLP_B_LOOKAHEAD;
   static_assert(LA >= 2 && LA <= 3 && LA <= G, "B ring has 4 entries");
   constexpr int HEAD_SLOTS = LA * TM;  // slots between the retiring barrier and the tile's end
@@ -273,6 +297,75 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
     }
   };
 
+  // ---- A3: separate load states for the two operands (the A loads run one tile ahead of the B
+  // loads), and the A ring's entries as byte offsets that rotate tile by tile.
+  constexpr int A_ENTRY = ATile::BYTES, A_RING = 3 * ATile::BYTES, B_ENTRY = NB * BTile::BYTES;
+  constexpr int LDA = ATile::PER_WAVE, LDB = NB * BTile::PER_WAVE;  // loads per wave and tile
+  uint32_t l3_soff[2] = {0, 0}, l3_event[2] = {0, 0};
+  uint64_t l3_head[2] = {0, 0};
+  int l3_cd[2] = {-1, -1};
+  bool l3_seg = false;
+  auto l3_start = [&]() __attribute__((always_inline)) {
+    load_state_start();
+    l3_soff[0] = ld_soff_a; l3_soff[1] = ld_soff_b;
+    l3_event[0] = ld_event_a; l3_event[1] = ld_event_b;
+    l3_head[0] = ld_head_a; l3_head[1] = ld_head_b;
+    l3_cd[0] = l3_cd[1] = ld_countdown;
+    l3_seg = ld_event_seg;
+  };
+  auto l3_advance = [&](int op) __attribute__((always_inline)) {
+    const bool fire = l3_cd[op] == 0;
+    const uint32_t nx = l3_soff[op] + (op == 0 ? a_step : b_step);
+    l3_soff[op] = fire ? l3_event[op] : nx;
+    l3_cd[op] -= 1;
+    if constexpr (NB == 1) {
+      const bool sw = fire && l3_seg;
+      l3_head[op] = sw ? rsrc_head(op == 0 ? ra[1] : rb[1]) : l3_head[op];
+    }
+  };
+  // Load z of a tile in issue order: the B loads first (z < LDB), then the A loads.
+  auto l3_is_b = [](int z) __attribute__((always_inline)) { return z < LDB; };
+  auto l3_index = [](int z) __attribute__((always_inline)) { return z < LDB ? z % BTile::PER_WAVE : z - LDB; };
+  auto l3_starts_group = [&](int z) __attribute__((always_inline)) { return (l3_index(z) & 3) == 0; };
+  // M0 for the group that load z starts; b_parity: ring entry of the B tile being filled,
+  // a_off: ring offset of the A tile being filled.
+  auto l3_base = [&](int z, int b_parity, uint32_t a_off) __attribute__((always_inline)) {
+    if (l3_is_b(z)) {
+      const int bsel = z / BTile::PER_WAVE, i = z % BTile::PER_WAVE;
+      set_lds_dma_base(lds_base + A_RING + b_parity * B_ENTRY + bsel * BTile::BYTES +
+                       (wave * BTile::PER_WAVE + i) * 1024);
+    } else {
+      set_lds_dma_base(lds_base + a_off + (wave * ATile::PER_WAVE + (z - LDB)) * 1024);
+    }
+  };
+  auto l3_issue = [&](int z) __attribute__((always_inline)) {
+    buffer_rsrc r;
+    uint32_t voff, soff;
+    if (l3_is_b(z)) {
+      const int bsel = z / BTile::PER_WAVE, i = z % BTile::PER_WAVE;
+      r = NB == 2 ? rb[bsel] : buffer_rsrc{(int)(uint32_t)l3_head[1], (int)(uint32_t)(l3_head[1] >> 32), rb[0][2], rb[0][3]};
+      voff = boff[i];
+      soff = l3_soff[1];
+    } else {
+      r = buffer_rsrc{(int)(uint32_t)l3_head[0], (int)(uint32_t)(l3_head[0] >> 32), ra[0][2], ra[0][3]};
+      voff = aoff[z - LDB];
+      soff = l3_soff[0];
+    }
+    switch (l3_index(z) & 3) {
+      case 0: load16_to_lds_at<0>(r, voff, soff); break;
+      case 1: load16_to_lds_at<1024>(r, voff, soff); break;
+      case 2: load16_to_lds_at<2048>(r, voff, soff); break;
+      default: load16_to_lds_at<3072>(r, voff, soff); break;
+    }
+  };
+  auto a3_next = [](uint32_t off) __attribute__((always_inline)) {
+    const uint32_t n = off + A_ENTRY;
+    return n == (uint32_t)A_RING ? 0u : n;
+  };
+  auto a3_prev = [](uint32_t off) __attribute__((always_inline)) {
+    return off == 0u ? (uint32_t)(A_RING - A_ENTRY) : off - A_ENTRY;
+  };
+
   vec8 af[2][TM];  // A fragments: bank = step parity
   vec8 bq[4];      // B fragment ring: entry = (step * G + group) % 4
   auto fetch_a = [&](int bank, int i, int kt, int ks) __attribute__((always_inline)) {
@@ -284,6 +377,15 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
     const int bsel = g / TN, j = g % TN;
     bq[entry] = BTile::template frag_mi<MI>(s + ATile::BYTES + bsel * BTile::BYTES,
                                             wn * WTN + j * MI, ks, lane);
+  };
+
+  auto fetch_a3 = [&](int bank, int i, uint32_t a_off, int ks) __attribute__((always_inline)) {
+    af[bank][i] = ATile::template frag_mi<MI>(smem + a_off, wm * WTM + i * MI, ks, lane);
+  };
+  auto fetch_b3 = [&](int entry, int g, int kt, int ks) __attribute__((always_inline)) {
+    const char* s = smem + A_RING + (kt & 1) * B_ENTRY;
+    const int bsel = g / TN, j = g % TN;
+    bq[entry] = BTile::template frag_mi<MI>(s + bsel * BTile::BYTES, wn * WTN + j * MI, ks, lane);
   };
 
   // One reduction tile.  NEXT: tile kt+1 exists.  The wavefront is alone on its SIMD: whatever
@@ -336,6 +438,68 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
             if (slot % LOAD_SLOTS == LOAD_PHASE && slot / LOAD_SLOTS < L) issue_one(slot / LOAD_SLOTS);
             const int nx = (slot + 1) / LOAD_SLOTS;
             if ((slot + 1) % LOAD_SLOTS == LOAD_PHASE && nx < L && starts_group(nx)) dma_base(lkt, nx);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  };
+
+  // The same for the A3 ring.  Slots are counted from the last barrier (the one in tile kt-1): it
+  // frees the B entry of tile kt-1, which takes tile kt+1, and the A entry of tile kt-1, which
+  // takes tile kt+2.  The LDA + LDB loads go out one per LSL slots, the B loads first (they must
+  // land by the barrier in tile kt), then the A loads (which have until the barrier in tile kt+1):
+  // the barrier in tile kt waits for everything but those LDA youngest loads.
+  auto tile_body3 = [&](int kt, auto next_c) __attribute__((always_inline)) {
+    constexpr bool NEXT = decltype(next_c)::value;
+    constexpr int L3 = LDA + LDB;
+    constexpr int LSL = TILE_SLOTS / L3, PH = LSL >= 4 ? 2 : 0;
+    static_assert(L3 * LSL <= TILE_SLOTS && LSL >= 1, "a tile's loads must fit a tile");
+    static_assert((LDB - 1) * LSL + PH < HEAD_SLOTS + (KSTEPS - 1) * G * TM + TM - 1, "last B load before the B state moves on");
+    static_assert(LDB * LSL >= HEAD_SLOTS, "A loads go out in the tile proper");
+    static_assert((L3 - 1) * LSL + PH < HEAD_SLOTS + (KSTEPS - 1) * G * TM + (G - LA - 1) * TM + TM - 1, "last A load before the A state moves on");
+    // (derived from the tile counter: a ring position carried from tile to tile as a variable of
+    // its own made the register allocator move accumulators around inside the loop)
+    const uint32_t a_rd = ((uint32_t)(kt - kt_first) % 3u) * (uint32_t)A_ENTRY;
+    const uint32_t a_nxt = a3_next(a_rd), a_fill = a3_prev(a_rd);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const bool last = ks == KSTEPS - 1;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool handover = last && g >= G - LA;
+        if (NEXT && last && g == G - LA) {
+          wait_vmem<LDA>();  // all but the A loads of the tile after next
+          __syncthreads();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          acc[g][i] = mfma_mi<T, MI>(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
+          if (i == 0) {
+            const int g2 = g + LA;
+            if (g2 < G) fetch_b3((ks * G + g2) % 4, g2, kt, ks);
+            else if (!last) fetch_b3(((ks + 1) * G + g2 - G) % 4, g2 - G, kt, ks + 1);
+            else if (NEXT) fetch_b3((g2 - G) % 4, g2 - G, kt + 1, 0);
+          }
+          if (!last) {
+            if (i == 1 && g < TM) fetch_a3((ks + 1) & 1, g, a_rd, ks + 1);
+          } else if (NEXT && handover) {
+            constexpr int AH = (TM + LA - 1) / LA;
+            const int h = (g - (G - LA)) * AH + (i - 1);
+            if (i >= 1 && i <= AH && h < TM) fetch_a3(0, h, a_nxt, 0);
+          }
+          if (NEXT) {
+            const int slot = handover ? (g - (G - LA)) * TM + i : HEAD_SLOTS + (ks * G + g) * TM + i;
+            // B entry being filled: behind this tile's barrier that of tile kt (with tile kt+2),
+            // before it that of tile kt-1 (with tile kt+1); A entry: a_fill, tile kt+2, always
+            // before the barrier.
+            const int b_parity = handover ? (kt & 1) : ((kt + 1) & 1);
+            if (slot % LSL == PH && slot / LSL < L3) l3_issue(slot / LSL);
+            const int nz = (slot + 1) / LSL;
+            if ((slot + 1) % LSL == PH && nz < L3 && l3_starts_group(nz)) l3_base(nz, b_parity, a_fill);
+            if (last && g == 0 && i == TM - 1) l3_advance(1);
+            if (last && g == G - LA - 1 && i == TM - 1) l3_advance(0);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -397,24 +561,61 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // issued (tile 0's own slots issue the rest); wait for tile 0.
   constexpr int HEAD_LOADS = (HEAD_SLOTS - LOAD_PHASE + LOAD_SLOTS - 1) / LOAD_SLOTS;
   constexpr int L_HEAD = HEAD_LOADS < L ? HEAD_LOADS : L;
-  load_state_start();
+  if constexpr (A3) {
+    constexpr int L3 = LDA + LDB, LSL3 = TILE_SLOTS / L3, PH3 = LSL3 >= 4 ? 2 : 0;
+    constexpr int HEAD_B = (HEAD_SLOTS - PH3 + LSL3 - 1) / LSL3 < LDB ? (HEAD_SLOTS - PH3 + LSL3 - 1) / LSL3 : LDB;
+    l3_start();
+    // tile 0 (A entry 0, B entry kt_first & 1), tile 1's A (entry 1) and the B loads of tile 1 that
+    // the handover slots of a tile before would have issued
 #pragma unroll
-  for (int x = 0; x < L; ++x) {
-    if (starts_group(x)) dma_base(kt_first, x);
-    issue_one(x);
+    for (int z = LDB; z < L3; ++z) {
+      if (l3_starts_group(z)) l3_base(z, 0, 0u);
+      l3_issue(z);
+    }
+#pragma unroll
+    for (int z = 0; z < LDB; ++z) {
+      if (l3_starts_group(z)) l3_base(z, kt_first & 1, 0u);
+      l3_issue(z);
+    }
+    l3_advance(0);
+    l3_advance(1);
+#pragma unroll
+    for (int z = LDB; z < L3; ++z) {
+      if (l3_starts_group(z)) l3_base(z, 0, (uint32_t)A_ENTRY);
+      l3_issue(z);
+    }
+#pragma unroll
+    for (int z = 0; z < HEAD_B; ++z) {
+      if (l3_starts_group(z)) l3_base(z, (kt_first + 1) & 1, 0u);
+      l3_issue(z);
+    }
+    l3_advance(0);
+    wait_vmem<LDA + HEAD_B>();
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fetch_a3(0, i, 0u, 0);
+#pragma unroll
+    for (int g = 0; g < LA; ++g) fetch_b3(g, g, kt_first, 0);
+  } else {
+    load_state_start();
+#pragma unroll
+    for (int x = 0; x < L; ++x) {
+      if (starts_group(x)) dma_base(kt_first, x);
+      issue_one(x);
+    }
+    load_state_advance();
+#pragma unroll
+    for (int x = 0; x < L_HEAD; ++x) {
+      if (starts_group(x)) dma_base(kt_first + 1, x);
+      issue_one(x);
+    }
+    wait_vmem<L_HEAD>();
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fetch_a(0, i, kt_first, 0);
+#pragma unroll
+    for (int g = 0; g < LA; ++g) fetch_b(g, g, kt_first, 0);
   }
-  load_state_advance();
-#pragma unroll
-  for (int x = 0; x < L_HEAD; ++x) {
-    if (starts_group(x)) dma_base(kt_first + 1, x);
-    issue_one(x);
-  }
-  wait_vmem<L_HEAD>();
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < TM; ++i) fetch_a(0, i, kt_first, 0);
-#pragma unroll
-  for (int g = 0; g < LA; ++g) fetch_b(g, g, kt_first, 0);
   __builtin_amdgcn_sched_barrier(0);
 
   // Epilogue work items of a wavefront: MI-row slab i of its tile, then (row, 8-column group)
@@ -438,7 +639,10 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   typename Epi::template Prefetch<8> pf[PD > 0 ? PD : 1];
 
   int kt = kt_first;
-  for (; kt + 1 < kt_total; ++kt) tile_body(kt, std::true_type{});
+  for (; kt + 1 < kt_total; ++kt) {
+    if constexpr (A3) tile_body3(kt, std::true_type{});
+    else tile_body(kt, std::true_type{});
+  }
   // (the operand fragments are still live during the last reduction tile: the first PD_EARLY
   // items are fetched before it, the rest of the PD behind it)
   constexpr int PD_EARLY = PD < 8 ? PD : 8;
@@ -450,7 +654,8 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
       Epi::template prefetch<8>(ea, min(m, ga.M - 1), min(n, ga.N - 8), pf[q]);
     }
   }
-  tile_body(kt, std::false_type{});
+  if constexpr (A3) tile_body3(kt, std::false_type{});
+  else tile_body(kt, std::false_type{});
   if (PD > PD_EARLY && !streamk) {
 #pragma unroll
     for (int q = PD_EARLY; q < PD; ++q) {
@@ -693,7 +898,7 @@ template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool 
           typename Epi>
 hipError_t launch_streamk_tail(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
   if constexpr (!Epi::SPLIT && MI == 16 && BM == 256) {
-    typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+    typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, wants_ring_a3<T, Epi>()> Cfg;
     constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi, true>;
     if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
     hipLaunchKernelGGL(kern, dim3(ga.sk_wgs), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, ga, ea);
@@ -726,7 +931,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
           typename Epi>
 hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
-  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, wants_ring_a3<T, Epi>()> Cfg;
   constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
   if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   const int splits = Epi::SPLIT ? ga.splits : 1;
@@ -743,7 +948,7 @@ hipError_t launch_gemm_pipelined(const GemmArgs& ga, const typename Epi::Args& e
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
           typename Epi>
 hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipStream_t s) {
-  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB> Cfg;
+  typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, wants_ring_a3<T, Epi>()> Cfg;
   constexpr auto kern = gemm_group_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>;
   if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
   int total = 0;
