@@ -90,12 +90,12 @@ struct PipeConfig {
   static constexpr int EPI_LD = WTN + 4;                                // fp32 staging row
   static constexpr int EPI_WAVE_BYTES = NB * MI * EPI_LD * 4;
   // A3: THREE ring entries of the A operand and two of the B operand(s), all of a workgroup's
-  // 160 KiB.  The A loads of a tile then have two tiles' time to land, so a tile's loads can be
+  // 160 KiB (80 KiB for the 128-row tiles: two workgroups per CU as before).  The A loads of a tile then have two tiles' time to land, so a tile's loads can be
   // spread evenly over the tile (B in its first half, A in its second) instead of going out back
   // to back at the rate the texture addresser can take at best, which is where a load that misses
   // L2 backs the queue up into the issuing wavefronts (down projection: queue-full stalls 166 -> 10
   // clocks per tile, 2664 -> 2451 clocks per tile, -4 % run time; input gradient -2 %).
-  static constexpr bool A3 = RING_A3 && BM == 256 && MI == 16 && !A_KS;
+  static constexpr bool A3 = RING_A3 && (BM == 256 || BM == 128) && MI == 16 && !A_KS;
   static constexpr int MAIN_BYTES = A3 ? 3 * ATile::BYTES + NS * NB * BTile::BYTES : NS * STAGE;
   static_assert(MAIN_BYTES <= 160 * 1024, "a workgroup has 160 KiB of LDS");
   static constexpr int LDS_BYTES = MAIN_BYTES > NW * EPI_WAVE_BYTES ? MAIN_BYTES : NW * EPI_WAVE_BYTES;
