@@ -48,6 +48,9 @@ DTYPE = torch.float16
 # whenever the weight-gradient kernels or their tile order change.
 DW_GROUP_TRAFFIC_BYTES = 5.22e9
 DW_GROUP_ALGORITHMIC_BYTES = 1.258e9  # dG, dU, dY, H once, x twice, three dW once
+# The same for one skinny-M forward at M=16, K=8192, N=28672 (both kernels):
+# profiles/decode_hbm_traffic_fp16_M16_K8192_N28672.txt.
+DECODE_TRAFFIC_BYTES = 1.469e9
 
 _flush_buf = None
 
@@ -270,7 +273,9 @@ def _config_lines(dev):
                 "bytes": nbytes, "gbps": _r(nbytes / t["p50"] / 1e6, 1), "tflops": _r(6.0 * m * n * k / t["p50"] / 1e9, 1),
                 "cache_flush_between_reps": True,
                 "roofline": {"bound": "hbm", "achieved": _r(nbytes / t["p50"] / 1e6, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                             "frac": _r(nbytes / t["p50"] / 1e6 / PEAK_HBM_GBPS)}},
+                             "frac": _r(nbytes / t["p50"] / 1e6 / PEAK_HBM_GBPS), "traffic": DECODE_TRAFFIC_BYTES,
+                             "traffic_note": "HBM-side bytes per forward from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                             "(profiles/decode_hbm_traffic_fp16_M16_K8192_N28672.txt)"}},
         "cpu": {"ms": _r(cpu_t * 1e3, 1), "gbps": _r(3 * k * cpu_n * 4 / cpu_t / 1e9, 1), "tflops": _r(cpu_tf, 4),
                 "sample": f"all 16 rows, intermediate columns 0..{cpu_n - 1} of {n} (fp32 weights: {3 * k * cpu_n * 4 / 1e6:.0f} MB), "
                           "fp32 torch-CPU oracle, median of 2 after 1 warm-up"},
