@@ -13,7 +13,7 @@
 #include "launch.hpp"
 
 #ifndef GMLP_MI
-#define GMLP_MI 16  // MFMA shape of the GEMM units (a build-wide knob: make EXTRA=-DGMLP_MI=32)
+#define GMLP_MI 16  // MFMA shape of the GEMM units (gemm_inst.hip accepts no other)
 #endif
 
 namespace {
