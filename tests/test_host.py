@@ -334,7 +334,19 @@ def test_m0_checker_flags_compiler_generated_m0_uses(tmp_path):
     bad_write = "_Z4kern:\n" + dma + "\ts_mov_b32 m0, s9\n\ts_endpgm\n"
     bad_use = "_Z4kern:\n" + dma + "\tv_movrels_b32_e32 v0, v1\n\ts_endpgm\n"
     other = "_Z5plain:\n\ts_mov_b32 m0, s9\n\ts_endpgm\n"
-    for text, expect in ((good, 0), (bad_write, 1), (bad_use, 1), (other, 0), (good + other, 0), (other + bad_write, 1)):
+    for text, expect in ((good, 0), (bad_write, 1), (bad_use, 1), (good + other, 0), (other + bad_write, 1)):
         f = tmp_path / "k.s"
         f.write_text(text)
         assert mod.check(str(f)) == expect
+    # A unit in which the scan recognises no kernel with such loads has verified nothing: that
+    # fails as well (kernel labels or inline-assembly markers the scan no longer matches), unless
+    # the caller says the file is expected to have none.
+    unmarked = "_Z4kern:\n\tbuffer_load_dwordx4 v1, s[8:11], s2 offen offset:1024 lds\n\ts_mov_b32 m0, s9\n\ts_endpgm\n"
+    relabelled = good.replace("_Z4kern:", "kern$local:")
+    for text in (other, unmarked, relabelled, ""):
+        f = tmp_path / "k.s"
+        f.write_text(text)
+        assert mod.check(str(f)) == 1
+        assert mod.check(str(f), minimum=0) == 0
+    f.write_text(good)
+    assert mod.check(str(f), minimum=2) == 1

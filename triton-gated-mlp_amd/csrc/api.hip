@@ -12,10 +12,6 @@
 
 #include "launch.hpp"
 
-#ifndef GMLP_MI
-#define GMLP_MI 16  // MFMA shape of the GEMM units (gemm_inst.hip accepts no other)
-#endif
-
 namespace {
 
 thread_local char g_err[512] = "";
@@ -199,7 +195,6 @@ struct StreamK {
 StreamK plan_streamk(int dtype, int64_t tiles, int64_t kt) {
   StreamK p;
   const int64_t cus = num_cu(), tail = tiles % cus;
-  if (GMLP_MI != 16) return p;  // the second stage knows the accumulator layout of the 16x16x32 MFMA only
   if (dtype == GMLP_F32 || tail == 0 || kt < 8) return p;
   if ((double)(cus - tail) / (double)cus * (double)kt <= 50.0) return p;
   int64_t wgs = tail * kt / 8;
@@ -273,7 +268,7 @@ int gmlp_init(void) {
   (void)num_cu();
   if (hipError_t e = gmlp::prepare_lds_kernels()) return hip_result(__func__, e);
   float* scratch = nullptr;
-  return hip_result(__func__, gmlp::colsum_static_scratch(&scratch));
+  return hip_result(__func__, gmlp::colsum_static_scratch(&scratch, nullptr));
 }
 
 size_t gmlp_workspace_bytes(int op, int64_t M, int64_t K, int64_t N, int dtype) {

@@ -157,13 +157,18 @@ template hipError_t launch_colsum_group<float>(const ColsumGroup<float>&, int, i
 // pointer hipGetSymbolAddress returned for the current device.
 static __device__ __align__(256) float scratch[(size_t)COLSUM_SPLITS * COLSUM_STATIC_MAX_C];
 
-hipError_t colsum_static_scratch(float** out) {
+hipError_t colsum_static_scratch(float** out, hipStream_t s) {
   static std::atomic<float*> known[64];  // per device
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   const bool tracked = dev >= 0 && dev < 64;
   float* p = tracked ? known[dev].load(std::memory_order_acquire) : nullptr;
   if (p == nullptr) {
+    // first use on this device (gmlp_init makes it ahead of time): a symbol lookup is not
+    // something to do while the stream is being captured
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipError_t e = hipStreamIsCapturing(s, &st)) return e;
+    if (st != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
     void* q = nullptr;
     if (hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch))) return e;
     if (q == nullptr) return hipErrorInvalidSymbol;
@@ -179,7 +184,7 @@ hipError_t colsum_static_scratch(float** out) {
 template <typename T>
 hipError_t launch_colsum_static(const T* a, T* out, int64_t M, int64_t C, hipStream_t s) {
   float* ws = nullptr;
-  if (hipError_t e = colsum_static_scratch(&ws)) return e;
+  if (hipError_t e = colsum_static_scratch(&ws, s)) return e;
   ColsumGroup<T> g = {};
   g.a[0] = a;
   g.out[0] = out;

@@ -10,7 +10,11 @@ inline-assembly LDS-DMA load, no instruction OUTSIDE the inline-assembly blocks 
 none may be of a kind that implies an M0 use the compiler chose (s_movrel*, v_movrel*, s_sendmsg,
 ds_gws_*).  A violation would send tiles to the wrong LDS address without any other symptom.
 
-usage: check_m0.py file.s      (exit status 1 on a violation)
+A file in which the scan recognises no kernel with such loads fails too (every GEMM unit has
+several): kernels are found by their mangled label and the loads by the inline-assembly markers,
+and a compiler that changed either would otherwise make the check pass without checking anything.
+
+usage: check_m0.py file.s [minimum kernels, default 1]     (exit status 1 on a violation)
 """
 import re
 import sys
@@ -20,7 +24,7 @@ USES_M0 = re.compile(r"^(s_movrel|v_movrel|s_sendmsg|ds_gws_)")
 LDS_DMA = re.compile(r"^buffer_load_\S+\s.*\blds\b")
 
 
-def check(path):
+def check(path, minimum=1):
     lines = open(path).read().split("\n")
     starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
     failures = 0
@@ -52,8 +56,12 @@ def check(path):
                 print(f"{path}:{line_no}: {name}: compiler-generated use of M0 in a kernel with LDS-DMA loads: {text}")
                 failures += 1
     print(f"check_m0: {checked} kernels with LDS-DMA loads checked in {path}, {failures} violation(s)")
+    if checked < minimum:
+        print(f"{path}: expected at least {minimum} kernel(s) with LDS-DMA loads, recognised {checked}: "
+              "the scan no longer matches the assembly, nothing was verified")
+        failures += 1
     return failures
 
 
 if __name__ == "__main__":
-    sys.exit(1 if check(sys.argv[1]) else 0)
+    sys.exit(1 if check(sys.argv[1], int(sys.argv[2]) if len(sys.argv) > 2 else 1) else 0)

@@ -66,9 +66,7 @@ constexpr int ds_part_buffers(int nmat, int mt, int segb) {
 }
 constexpr uint32_t DS_NOWHERE = 0x80000000u;  // voffset beyond any operand (operands are < 2 GiB)
 constexpr int DS_WIDE_SEGMENT_MAX_M = 20;     // two token tiles: 512-byte row segments up to here, 256 beyond
-#ifndef GMLP_DECODE_TILED_MIN
-#define GMLP_DECODE_TILED_MIN 10
-#endif
+constexpr int DS_H_TILED_MIN_M = 10;           // H goes out in fragment order above this many token rows
 
 struct StreamArgs {
   const void* x;      // [M, ldx] token rows (x or H)
@@ -389,7 +387,7 @@ static hipError_t launch_stream(const StreamArgs& a, int num_cu, hipStream_t s) 
 // Layout of the intermediate H between the two kernels.  Row-major [M, N] costs the down projection
 // M pieces of 64 bytes per token-operand fragment, fragment order always one KiB (16 token slots):
 // cheaper from about half-full upwards.  Two token tiles always use fragment order.
-static int ds_h_tiled(int M) { return M > GMLP_DECODE_TILED_MIN ? 1 : 0; }
+static int ds_h_tiled(int M) { return M > DS_H_TILED_MIN_M ? 1 : 0; }
 
 bool decode_stream_supported(int M, int K, int N) {
   return M >= 1 && M <= 32 && K % DS_CH == 0 && N % DS_CH == 0 && K >= DS_WAVES * DS_CH && N >= DS_WAVES * DS_CH &&

@@ -570,10 +570,8 @@ struct EpiDh {
   }
   // G and U come from HBM and every workgroup of a round reaches its epilogue at about the same
   // time; a kernel that can, fetches them this many W-wide items ahead of their use.
-#ifndef GMLP_DH_PREFETCH
-#define GMLP_DH_PREFETCH 8
-#endif
-  static constexpr int PREFETCH_DEPTH = GMLP_DH_PREFETCH;
+  // (8 W-wide items; 12 and 16 measured the same)
+  static constexpr int PREFETCH_DEPTH = 8;
   template <int W>
   struct Prefetch {
     typename PackW<T, W>::type g, u;

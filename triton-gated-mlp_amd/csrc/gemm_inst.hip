@@ -11,20 +11,14 @@ typedef f16 DT;
 typedef bf16 DT;
 #endif
 
-#ifndef GMLP_MI
-#define GMLP_MI 16  // MFMA shape: v_mfma_f32_16x16x32
-#endif
-#if GMLP_MI != 16
-#error "the GEMM units are maintained for the 16x16x32 MFMA only (the 32x32x16 instance of the loop was 3-5 % slower when both were measured and has not followed the kernel since)"
-#endif
 #define GMLP_LARGE(AKS, BKS, NB, EPI, BN_L) \
-  launch_gemm_pipelined<DT, 256, BN_L, GMLP_MI, 2, 2, AKS, BKS, NB, EPI<DT>>
+  launch_gemm_pipelined<DT, 256, BN_L, 16, 2, 2, AKS, BKS, NB, EPI<DT>>
 #define GMLP_MEDIUM(AKS, BKS, NB, EPI, BN_M) \
-  launch_gemm_pipelined<DT, 128, BN_M, GMLP_MI, 2, 2, AKS, BKS, NB, EPI<DT>>
+  launch_gemm_pipelined<DT, 128, BN_M, 16, 2, 2, AKS, BKS, NB, EPI<DT>>
 #define GMLP_LARGE_GROUP \
-  launch_gemm_group_pipelined<DT, 256, 256, GMLP_MI, 2, 2, true, true, 1, EpiStore<DT>>
+  launch_gemm_group_pipelined<DT, 256, 256, 16, 2, 2, true, true, 1, EpiStore<DT>>
 #define GMLP_MEDIUM_GROUP \
-  launch_gemm_group_pipelined<DT, 128, 128, GMLP_MI, 2, 2, true, true, 1, EpiStore<DT>>
+  launch_gemm_group_pipelined<DT, 128, 128, 16, 2, 2, true, true, 1, EpiStore<DT>>
 
 #define GMLP_DISPATCH(AKS, BKS, NB, EPI, BN_L, BN_M)                                             \
   if (tile_class == TILE_LARGE) return GMLP_LARGE(AKS, BKS, NB, EPI, BN_L)(ga, ea, s);           \
@@ -44,7 +38,7 @@ hipError_t launch_gateup<DT>(int tile_class, const GemmArgs& ga, const EpiGateUp
 }
 template <>
 hipError_t launch_gateup_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
-  return launch_gemm_pipelined<DT, 128, 64, GMLP_MI, 2, 2, false, false, 2, EpiPartial<DT>>(ga, ea, s);
+  return launch_gemm_pipelined<DT, 128, 64, 16, 2, 2, false, false, 2, EpiPartial<DT>>(ga, ea, s);
 }
 #elif GMLP_KIND == 1
 template <>
@@ -54,7 +48,7 @@ hipError_t launch_linear<DT>(int tile_class, const GemmArgs& ga, const EpiStore<
 }
 template <>
 hipError_t launch_linear_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
-  return launch_gemm_pipelined<DT, 128, 128, GMLP_MI, 2, 2, false, false, 1, EpiPartial<DT>>(ga, ea, s);
+  return launch_gemm_pipelined<DT, 128, 128, 16, 2, 2, false, false, 1, EpiPartial<DT>>(ga, ea, s);
 }
 #elif GMLP_KIND == 2
 template <>
@@ -70,7 +64,7 @@ hipError_t launch_dx<DT>(int tile_class, const GemmArgs& ga, const EpiStore<DT>:
 }
 template <>
 hipError_t launch_dx_split<DT>(const GemmArgs& ga, const EpiPartial<DT>::Args& ea, hipStream_t s) {
-  return launch_gemm_pipelined<DT, 128, 128, GMLP_MI, 2, 2, false, true, 1, EpiPartial<DT>>(ga, ea, s);
+  return launch_gemm_pipelined<DT, 128, 128, 16, 2, 2, false, true, 1, EpiPartial<DT>>(ga, ea, s);
 }
 #elif GMLP_KIND == 4
 template <>

@@ -38,27 +38,10 @@
 
 namespace gmlp {
 
-#ifndef GMLP_LOAD_CYCLES
-#define GMLP_LOAD_CYCLES 64  // one global->LDS load per this many MFMA cycles
-#endif
-#ifndef GMLP_B_LOOKAHEAD
-#define GMLP_B_LOOKAHEAD 3  // MFMA groups between the fetch of a B fragment and its use (2 or 3)
-#endif
-
-template <int MI>
-struct AccType;
-template <>
-struct AccType<32> { typedef f32x16 type; };
-template <>
-struct AccType<16> { typedef f32x4 type; };
-
-template <typename T, int MI>
-__device__ __forceinline__ typename AccType<MI>::type mfma_mi(typename Traits<T>::vec8 a,
-                                                              typename Traits<T>::vec8 b,
-                                                              typename AccType<MI>::type c) {
-  if constexpr (MI == 32) return Traits<T>::mfma(a, b, c);
-  else return Traits<T>::mfma16(a, b, c);
-}
+// Two-entry ring: one global->LDS load per this many MFMA cycles (32, 96 and 128 measured slower).
+constexpr int LOAD_CYCLES = 64;
+// MFMA groups between the fetch of a B fragment and its use (2 measured 0.3 % slower).
+constexpr int B_LOOKAHEAD = 3;
 
 // Kernels that get the three-entry A ring (see PipeConfig::A3): those with a reduction-contiguous A
 // operand other than dH, i.e. gate/up, the down projection and the input gradient.  The long
@@ -67,22 +50,19 @@ __device__ __forceinline__ typename AccType<MI>::type mfma_mi(typename Traits<T>
 // gradients' two transposed operands leave no registers for it (spills when tried).
 template <typename T, typename Epi>
 constexpr bool wants_ring_a3() {
-#ifdef GMLP_NO_RING_A3
-  return false;
-#else
   return !std::is_same<Epi, EpiDh<T>>::value;
-#endif
 }
 
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB, bool RING_A3 = false>
 struct PipeConfig {
+  static_assert(MI == 16, "the loop is written for v_mfma_f32_16x16x32 (4 accumulator floats per lane)");
   static constexpr int BK = 64, NS = 2;
   static constexpr int NW = WGM * WGN;
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;
   static constexpr int TM = WTM / MI, TN = WTN / MI, G = NB * TN;
   static constexpr int KF = 512 / MI;            // reduction elements per MFMA
   static constexpr int KSTEPS = BK / KF;
-  static constexpr int MFMA_CYCLES = MI == 32 ? 32 : 16;
+  static constexpr int MFMA_CYCLES = 16;
   typedef LdsTile<T, BM, BK, A_KS, NW> ATile;
   typedef LdsTile<T, BN, BK, B_KS, NW> BTile;
   static constexpr int STAGE = ATile::BYTES + NB * BTile::BYTES;
@@ -95,7 +75,7 @@ struct PipeConfig {
   // to back at the rate the texture addresser can take at best, which is where a load that misses
   // L2 backs the queue up into the issuing wavefronts (down projection: queue-full stalls 166 -> 10
   // clocks per tile, 2664 -> 2451 clocks per tile, -4 % run time; input gradient -2 %).
-  static constexpr bool A3 = RING_A3 && (BM == 256 || BM == 128) && MI == 16 && !A_KS;
+  static constexpr bool A3 = RING_A3 && (BM == 256 || BM == 128) && !A_KS;
   static constexpr int MAIN_BYTES = A3 ? 3 * ATile::BYTES + NS * NB * BTile::BYTES : NS * STAGE;
   static_assert(MAIN_BYTES <= 160 * 1024, "a workgroup has 160 KiB of LDS");
   static constexpr int LDS_BYTES = MAIN_BYTES > NW * EPI_WAVE_BYTES ? MAIN_BYTES : NW * EPI_WAVE_BYTES;
@@ -114,14 +94,14 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   typedef typename Cfg::ATile ATile;
   typedef typename Cfg::BTile BTile;
   typedef typename Traits<T>::vec8 vec8;
-  typedef typename AccType<MI>::type acc_t;
+  typedef f32x4 acc_t;
   constexpr int BK = Cfg::BK, NS = Cfg::NS;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, G = Cfg::G, WTM = Cfg::WTM, WTN = Cfg::WTN;
   constexpr int KSTEPS = Cfg::KSTEPS, STAGE = Cfg::STAGE, L = Cfg::LOADS;
-  constexpr int LOAD_SLOTS = GMLP_LOAD_CYCLES / Cfg::MFMA_CYCLES;  // MFMA slots per load
+  constexpr int LOAD_SLOTS = LOAD_CYCLES / Cfg::MFMA_CYCLES;  // MFMA slots per load
   constexpr int TILE_SLOTS = KSTEPS * G * TM;                         // MFMA slots per tile
   constexpr bool A3 = Cfg::A3;
-  constexpr int LA = GMLP_B_LOOKAHEAD;
+  constexpr int LA = B_LOOKAHEAD;
   static_assert(LA >= 2 && LA <= 3 && LA <= G, "B ring has 4 entries");
   constexpr int HEAD_SLOTS = LA * TM;  // slots between the retiring barrier and the tile's end
   // Fragment fetches sit in slots 0 and 1 of a group; with four or more slots per load the loads
@@ -410,7 +390,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          acc[g][i] = mfma_mi<T, MI>(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
+          acc[g][i] = Traits<T>::mfma16(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
           // --- B fragment of the group LA ahead
           if (i == 0) {
             const int g2 = g + LA;
@@ -475,7 +455,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          acc[g][i] = mfma_mi<T, MI>(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
+          acc[g][i] = Traits<T>::mfma16(bq[(ks * G + g) % 4], af[ks & 1][i], acc[g][i]);
           if (i == 0) {
             const int g2 = g + LA;
             if (g2 < G) fetch_b3((ks * G + g2) % 4, g2, kt, ks);
@@ -625,9 +605,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // are dropped when it comes to storing.
   constexpr int ITEMS = MI * WTN / 8 / 64;  // items per lane and slab
   constexpr int NITEMS = TM * ITEMS;
-  // (the 32x32x16 instance has fewer registers to spare; the depth hardly matters, 4 = 8 = 12 measured)
-  constexpr int PD_WANTED = MI == 32 && Epi::PREFETCH_DEPTH > 4 ? 4 : Epi::PREFETCH_DEPTH;
-  constexpr int PD = PD_WANTED < NITEMS ? PD_WANTED : NITEMS;
+  constexpr int PD = Epi::PREFETCH_DEPTH < NITEMS ? Epi::PREFETCH_DEPTH : NITEMS;
   static_assert(MI * WTN / 8 % 64 == 0, "slab items must divide over the lanes");
   auto item_pos = [&](int q, int& row, int& m, int& n, int& cg) __attribute__((always_inline)) {
     int i = q / ITEMS, item = (q % ITEMS) * 64 + lane;
@@ -681,7 +659,6 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   constexpr int ELD = Cfg::EPI_LD;
   float* stg = (float*)(smem + wave * Cfg::EPI_WAVE_BYTES);
   const int mrow = lane & (MI - 1), nsub = 4 * (lane / MI);
-  constexpr int NV = MI == 32 ? 4 : 1;  // 4-column vectors a lane holds per accumulator
   // The slab loop exists once per activation the epilogue offers, each with the activation fixed
   // at compile time: a run-time switch inside the loop would leave every path threading its way
   // through several times its own code (measured: +7 % for relu to +30 % for gelu on the kernel).
@@ -692,14 +669,9 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const int b = g / TN, j = g % TN;
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-          f32x4 o;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = acc[g][i][4 * v + r];
-          if (streamk) *(f32x4*)(sk_slot + (size_t)(g * TM + i) * 64 * AV + 4 * v) = o;
-          else *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + 8 * v + nsub) = o;
-        }
+        const f32x4 o = acc[g][i];
+        if (streamk) *(f32x4*)(sk_slot + (size_t)(g * TM + i) * 64 * AV) = o;
+        else *(f32x4*)(stg + (b * MI + mrow) * ELD + j * MI + nsub) = o;
       }
       if (streamk) continue;
       // Same-wavefront LDS writes and reads are ordered; no barrier needed for a private slab.
@@ -717,22 +689,12 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
           *(f32x4*)v1 = *(const f32x4*)p1;
           *(f32x4*)(v1 + 4) = *(const f32x4*)(p1 + 4);
         }
-#ifdef GMLP_PREFETCH_FIRST
-        const typename Epi::template Prefetch<8> cur = pf[q % (PD > 0 ? PD : 1)];
-        if (q + PD < NITEMS) {
-          int row2, m2, n2, cg2;
-          item_pos(q + PD, row2, m2, n2, cg2);
-          Epi::template prefetch<8>(ea, min(m2, ga.M - 1), min(n2, ga.N - 8), pf[q % (PD > 0 ? PD : 1)]);
-        }
-        if (m < ga.M && n < ga.N) Epi::template apply<8, ACT>(ea, m, n, v0, v1, cur);
-#else
         if (m < ga.M && n < ga.N) Epi::template apply<8, ACT>(ea, m, n, v0, v1, pf[q % (PD > 0 ? PD : 1)]);
         if (q + PD < NITEMS) {
           int row2, m2, n2, cg2;
           item_pos(q + PD, row2, m2, n2, cg2);
           Epi::template prefetch<8>(ea, min(m2, ga.M - 1), min(n2, ga.N - 8), pf[q % (PD > 0 ? PD : 1)]);
         }
-#endif
       }
     }
   };
@@ -744,7 +706,7 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
   // Staging of a wavefront: planes x [16 rows][WTN elements], row r's 8-byte unit u stored at
   // u ^ 2 (r >> SH): the 32 lanes of a half-wave write (16 rows x 2 units) hit 64 distinct banks,
   // and a 16-byte read of chunk c of row r finds it at c ^ (r >> SH), 16 lanes covering all banks.
-  if constexpr (MI == 16 && Epi::PACKED) {
+  if constexpr (Epi::PACKED) {
     typedef typename PackW<T, 4>::type vec4;
     constexpr int P = Epi::PLANES;
     constexpr int UPR = WTN / 4;                       // 8-byte units per staging row
@@ -832,7 +794,6 @@ __device__ __forceinline__ void gemm_pipelined_body(const GemmArgs& ga, const ty
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, int NB, typename Epi>
 __global__ void __launch_bounds__(WGM* WGN * 64) streamk_fixup_kernel(GemmArgs ga, typename Epi::Args ea) {
   typedef PipeConfig<T, BM, BN, MI, WGM, WGN, false, false, NB> Cfg;
-  static_assert(MI == 16, "accumulator layout of the 16x16x32 MFMA");
   constexpr int TM = Cfg::TM, TN = Cfg::TN, G = Cfg::G, WTM = Cfg::WTM, WTN = Cfg::WTN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -897,7 +858,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64)
 template <typename T, int BM, int BN, int MI, int WGM, int WGN, bool A_KS, bool B_KS, int NB,
           typename Epi>
 hipError_t launch_streamk_tail(const GemmArgs& ga, const typename Epi::Args& ea, hipStream_t s) {
-  if constexpr (!Epi::SPLIT && MI == 16 && BM == 256) {
+  if constexpr (!Epi::SPLIT && BM == 256) {
     typedef PipeConfig<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, wants_ring_a3<T, Epi>()> Cfg;
     constexpr auto kern = gemm_kernel_pipelined<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi, true>;
     if (hipError_t e = allow_dynamic_lds(lds_kernel_of<kern, Cfg::LDS_BYTES>, s)) return e;
@@ -958,8 +919,10 @@ hipError_t launch_gemm_group_pipelined(GemmGroup<typename Epi::Args>& grp, hipSt
     total += tiles - grp.ga[g].sk_tiles;
   }
   for (int g = grp.count; g <= GEMM_GROUP_MAX; ++g) grp.first[g] = total;
-  hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);
-  if (hipError_t e = hipGetLastError()) return e;
+  if (total > 0) {  // (stream-K may have taken every tile of a single problem)
+    hipLaunchKernelGGL(kern, dim3(total), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, grp);
+    if (hipError_t e = hipGetLastError()) return e;
+  }
   for (int g = 0; g < grp.count; ++g) {
     if (grp.ga[g].sk_tiles <= 0) continue;
     if (hipError_t e = launch_streamk_tail<T, BM, BN, MI, WGM, WGN, A_KS, B_KS, NB, Epi>(grp.ga[g], grp.ea[g], s)) return e;

@@ -54,12 +54,12 @@ struct LdsTile {
     }
   }
 
-  // MFMA operand fragment (8 reduction elements per lane) for an MI x MI x (512/MI) instruction:
-  // rows row0 .. row0+MI-1, reduction step ks (512/MI elements).  Lane l carries row l % MI and
-  // reduction slots 8*(l / MI) .. +7.
+  // MFMA operand fragment (8 reduction elements per lane) for a 16 x 16 x 32 instruction: rows
+  // row0 .. row0+15, reduction step ks (32 elements).  Lane l carries row l % 16 and reduction
+  // slots 8*(l / 16) .. +7.
   template <int MI>
   static __device__ __forceinline__ vec8 frag_mi(const char* lds_tile, int row0, int ks, int lane) {
-    static_assert(MI == 16 || MI == 32, "MFMA tile is 16x16x32 or 32x32x16");
+    static_assert(MI == 16, "MFMA tile is 16x16x32");
     constexpr int CPS = 64 / MI;  // 16-byte chunks per row per reduction step
     if constexpr (!KS) {
       int row = row0 + (lane & (MI - 1));
@@ -70,8 +70,8 @@ struct LdsTile {
       // (kb+0..3, kb+4..7): lane r of the group addresses reduction row kb + r/4, rows
       // nb + 4*(r%4) .. +3, and receives the 4 reduction elements of row nb + r.
       int g = lane >> 4, r = lane & 15;
-      int nb = MI == 32 ? row0 + 16 * (g & 1) : row0;
-      int kb = MI == 32 ? ks * 16 + 8 * (g >> 1) : ks * 32 + 8 * g;
+      int nb = row0;
+      int kb = ks * 32 + 8 * g;
       int n = nb + 4 * (r & 3);
       int kq = r >> 2;  // == reduction row & 3
       int c = (n >> 3) ^ (4 * kq);

@@ -90,7 +90,9 @@ size_t colsum_workspace_bytes(int64_t M, int64_t C);
 // Column sums of one array with the first stage's partial sums in a static device array of the
 // library (no workspace argument, no allocation); C <= COLSUM_STATIC_MAX_C.
 constexpr int64_t COLSUM_STATIC_MAX_C = 32768;
-hipError_t colsum_static_scratch(float** out);  // address of that array on the current device
+// Address of that array on the current device; the first call on a device looks the symbol up
+// and refuses to while `s` is capturing.
+hipError_t colsum_static_scratch(float** out, hipStream_t s);
 template <typename T>
 hipError_t launch_colsum_static(const T* a, T* out, int64_t M, int64_t C, hipStream_t s);
 hipError_t launch_dropout_mask(uint8_t* mask, int64_t M, int64_t N, const DropoutParams& d,
