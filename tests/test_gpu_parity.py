@@ -1,7 +1,14 @@
 """Parity of the HIP path (through the C ABI) against the CPU oracle on identical seeded inputs.
 
-Tolerance: rtol = atol = 2e-2 element-wise for fp16/bf16 storage with fp32 accumulation, against
-the oracle evaluated in fp32 on the same (already rounded) inputs.
+Tolerance, one rule for every comparison in this file (`_close`): rtol = 2e-2 element-wise against the
+reference evaluated in fp32 on the same (already rounded) inputs, atol = 2e-2 * max(1, mean|ref|), and a
+relative Frobenius error below 1e-2.  The absolute term follows the magnitude of the tensor because
+an element's rounding error is set by the size of the terms that were summed (which is what
+mean|ref| measures), not by the element's own value: an element of a weight gradient that happens
+to come out near zero from 8192 products of size 1 cannot be held to 2e-2 of itself.  For outputs
+of typical size below one (Y, dX, G, U, H, dG, dU with the stated input distributions) the rule is
+the plain rtol = atol = 2e-2.  `test_cfg3_fp16_forward_backward_llama3_8b` holds the rule against a
+yardstick: torch's own fp16 module on the same inputs against the same oracle.
 """
 
 import contextlib
@@ -24,16 +31,16 @@ def _dev():
     return torch.device("cuda", 0)
 
 
-def _close(name, got, ref, rtol=RTOL, atol=ATOL):
+def _close(name, got, ref):
     got = got.detach().float().cpu()
     ref = ref.detach().float().cpu()
     assert got.shape == ref.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
     err = (got - ref).abs()
-    bound = atol + rtol * ref.abs()
-    bad = err > bound
+    atol = ATOL * max(1.0, ref.abs().mean().item() if ref.numel() else 0.0)
+    bad = err > atol + RTOL * ref.abs()
     rel_fro = ((got - ref).norm() / ref.norm().clamp_min(1e-30)).item()
-    # elements outside the plain band, whatever absolute tolerance the caller scaled up to
+    # elements outside the plain band, whatever the magnitude of the tensor scaled the absolute term to
     plain = int((err > ATOL + RTOL * ref.abs()).sum()) if err.numel() else 0
     print(
         f"  {name}: max_abs_err={err.max().item() if err.numel() else 0.0:.3e} rel_fro={rel_fro:.3e} "
@@ -41,7 +48,7 @@ def _close(name, got, ref, rtol=RTOL, atol=ATOL):
         flush=True,
     )
     assert not bad.any(), (
-        f"{name}: {int(bad.sum())} of {bad.numel()} elements outside rtol={rtol}, atol={atol}; "
+        f"{name}: {int(bad.sum())} of {bad.numel()} elements outside rtol={RTOL}, atol={atol:.3g}; "
         f"max_abs_err={err.max().item():.4e}, rel_fro={rel_fro:.3e}"
     )
     assert rel_fro < 1e-2, f"{name}: relative Frobenius error {rel_fro:.3e}"
@@ -107,9 +114,7 @@ def _run_module_case(c: Case, lean: bool = False, yardstick: bool = False):
     )
     _close("Y", y, ref["Y"])
     for n, g in zip(names, grads):
-        # weight gradients sum M terms: scale the absolute tolerance with the magnitude of the result
-        scale = max(1.0, ref[n].abs().mean().item())
-        _close(n, g, ref[n], atol=ATOL * scale)
+        _close(n, g, ref[n])
     if yardstick:
         from triton_gated_mlp import EagerGatedMLP, copy_weights
 
@@ -314,8 +319,8 @@ def test_other_activations_operator_level(act):
     hb = oracle.hidden_backward(dH.float(), f["G"], f["U"], act=act)
     _close("H", h, f["H"])
     _close("dX", dx, hb["dU"] @ o["W_up"] + hb["dG"] @ o["W_gate"])
-    _close("dW_up", dWu, hb["dU"].T @ o["x"], atol=ATOL * max(1.0, (hb["dU"].T @ o["x"]).abs().mean().item()))
-    _close("dW_gate", dWg, hb["dG"].T @ o["x"], atol=ATOL * max(1.0, (hb["dG"].T @ o["x"]).abs().mean().item()))
+    _close("dW_up", dWu, hb["dU"].T @ o["x"])
+    _close("dW_gate", dWg, hb["dG"].T @ o["x"])
 
 
 def test_device_activation_functions_against_float64_closed_forms():
@@ -380,9 +385,9 @@ def test_operator_level_fwd_bwd_match_closed_form():
     _close("hidden", h, ref["H"])
     dx, dW_up, dW_gp = mlp_hidden_states_bwd(x.to(dev), W_up.to(dev), W_gp.to(dev), dH.to(dev))
     hb = oracle.hidden_backward(dH.float(), ref["G"], ref["U"])
-    _close("dx", dx, hb["dU"] @ W_up.float() + hb["dG"] @ W_gp.float(), atol=ATOL * 4)
-    _close("dW_up", dW_up, hb["dU"].T @ x.float(), atol=ATOL * 4)
-    _close("dW_gp", dW_gp, hb["dG"].T @ x.float(), atol=ATOL * 4)
+    _close("dx", dx, hb["dU"] @ W_up.float() + hb["dG"] @ W_gp.float())
+    _close("dW_up", dW_up, hb["dU"].T @ x.float())
+    _close("dW_gp", dW_gp, hb["dG"].T @ x.float())
 
 
 def test_autograd_function_reference_signature():
@@ -711,7 +716,7 @@ def test_non_contiguous_inputs_and_partial_gradients():
     ref = oracle.backward(f(xw), f(mlp.gate_proj.weight), None, f(mlp.up_proj.weight), None, f(mlp.down_proj.weight),
                           None, f(dy))
     for n, got in zip(("dW_gate", "dW_up", "dW_down"), gw):
-        _close(n, got, ref[n], atol=ATOL * 4)
+        _close(n, got, ref[n])
 
 
 def test_many_tokens_tall_shape():
@@ -877,7 +882,7 @@ def test_streamk_seams_every_gemm_kind_against_fp32_matmul():
     lhs, rhs = rnd(Mred, R), rnd(Mred, C)
     dw = ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev))
     assert torch.equal(dw, ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev)))
-    _close("dW stream-K", dw, f(lhs).T @ f(rhs), atol=ATOL * 40)
+    _close("dW stream-K", dw, f(lhs).T @ f(rhs))
 
     # dW, grouped: 64 + 64 + 256 = 384 tiles (1.5 rounds); the shared-out tiles are the last 128 of
     # the last problem (reduction of 102 tiles: half a round saved is worth the second launch)
@@ -888,22 +893,100 @@ def test_streamk_seams_every_gemm_kind_against_fp32_matmul():
     outs2 = ops_bwd.dw_bwd_grouped(dev_pairs)
     for (a_, b_), got, again in zip(pairs, outs, outs2):
         assert torch.equal(got, again)
-        _close("dW grouped stream-K", got, f(a_).T @ f(b_), atol=ATOL * 40)
+        _close("dW grouped stream-K", got, f(a_).T @ f(b_))
+
+
+def test_streamk_pieces_that_straddle_tiles_every_gemm_kind():
+    """352 large tiles = one whole round and 96 tiles: 96 does not divide 256, so the shared-out
+    tiles go to 256 workgroups as even ranges of (tile, reduction tile) pairs that begin and end
+    inside tiles (the multi-piece loop, slot = workgroup + tile, the search for a tile's first
+    workgroup in the second stage).  Every kind of GEMM: two accumulator sets (gate/up), the dH
+    epilogue with its prefetch, a piece crossing the seam between dX's two reduction segments, both
+    operands reduction-strided with a ragged reduction (dW); against fp32 products on the host."""
+    from triton_gated_mlp import _cabi
+    from triton_gated_mlp.ops import bwd as ops_bwd
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(23)
+    rnd = lambda *shape, s=1.0: (s * torch.randn(*shape, generator=g)).half()
+    f = lambda t: t.float()
+    straddling = (96 + 256) * 65536 * 4  # slots of a plan without whole pieces per tile
+
+    M, K, N = 2048, 5184, 5632  # gate/up: 8 x 44 tiles of 256 x 128, 81 reduction tiles
+    assert _streamk_expected(_cabi.GMLP_OP_GATEUP_FWD, M, K, N) == straddling
+    x, wg, wu, bg = rnd(M, K), rnd(N, K, s=0.02), rnd(N, K, s=0.02), rnd(N, s=0.1)
+    hs = ops_fwd.gateup_fwd(x.to(dev), wg.to(dev), bg.to(dev), wu.to(dev), None, save_activations=True)
+    hs2 = ops_fwd.gateup_fwd(x.to(dev), wg.to(dev), bg.to(dev), wu.to(dev), None, save_activations=True)
+    assert torch.equal(hs.hidden, hs2.hidden) and torch.equal(hs.gate, hs2.gate) and torch.equal(hs.up, hs2.up)
+    ref = oracle.hidden_forward(f(x), f(wg), f(bg), f(wu), None, None, 0.0)
+    _close("gate/up straddling H", hs.hidden, ref["H"])
+    _close("gate/up straddling G", hs.gate, ref["G"])
+    _close("gate/up straddling U", hs.up, ref["U"])
+
+    M, K, N = 2048, 5184, 11264  # dH: 8 x 44 tiles of 256 x 256
+    assert _streamk_expected(_cabi.GMLP_OP_DH_BWD, M, K, N) == straddling
+    dy, wdn, G, U = rnd(M, K), rnd(K, N, s=0.02), rnd(M, N), rnd(M, N)
+    dg, du = ops_bwd.dh_bwd(dy.to(dev), wdn.to(dev), G.to(dev), U.to(dev))
+    dg2, du2 = ops_bwd.dh_bwd(dy.to(dev), wdn.to(dev), G.to(dev), U.to(dev))
+    assert torch.equal(dg, dg2) and torch.equal(du, du2)
+    hb = oracle.hidden_backward(f(dy) @ f(wdn), f(G), f(U), None, 0.0)
+    _close("dH straddling dG", dg, hb["dG"])
+    _close("dH straddling dU", du, hb["dU"])
+
+    M, K, N = 2048, 11264, 2624  # dX: two segments of 41 reduction tiles; pieces of 30-31 cross the seam
+    assert _streamk_expected(_cabi.GMLP_OP_DX_BWD, M, K, N) == straddling
+    dgv, duv, wg, wu = rnd(M, N), rnd(M, N), rnd(N, K, s=0.02), rnd(N, K, s=0.02)
+    dx = ops_bwd.dx_bwd(dgv.to(dev), duv.to(dev), wg.to(dev), wu.to(dev))
+    assert torch.equal(dx, ops_bwd.dx_bwd(dgv.to(dev), duv.to(dev), wg.to(dev), wu.to(dev)))
+    _close("dX straddling", dx, f(dgv) @ f(wg) + f(duv) @ f(wu))
+
+    Mred, R, C = 5192, 2048, 11264  # dW: 82 reduction tiles, the last one of 8 rows
+    assert _streamk_expected(_cabi.GMLP_OP_DW_BWD, Mred, R, C) == straddling
+    lhs, rhs = rnd(Mred, R), rnd(Mred, C)
+    dw = ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev))
+    assert torch.equal(dw, ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev)))
+    _close("dW straddling", dw, f(lhs).T @ f(rhs))
+
+
+def test_grouped_launch_of_one_problem_whose_tiles_all_go_to_streamk():
+    """A single weight gradient of 200 large tiles with a long reduction: fewer tiles than compute
+    units, so the plan shares out every tile and the grouped launch has no whole-tile grid left to
+    run (which must not be launched empty).  Against the fp32 product and gmlp_dw_bwd."""
+    import ctypes
+
+    from triton_gated_mlp import _cabi
+    from triton_gated_mlp.ops import bwd as ops_bwd
+
+    dev = _dev()
+    Mred, R, C = 16384, 2560, 5120
+    RC = (ctypes.c_int64 * 1)
+    nbytes = _cabi.lib().gmlp_dw_bwd_grouped_workspace_bytes(
+        1, Mred, ctypes.cast(RC(R), ctypes.c_void_p), ctypes.cast(RC(C), ctypes.c_void_p), 0)
+    assert nbytes == (200 + 256) * 65536 * 4  # all 200 tiles shared out over 256 workgroups
+    g = torch.Generator().manual_seed(29)
+    lhs = torch.randn(Mred, R, generator=g).half()
+    rhs = torch.randn(Mred, C, generator=g).half()
+    (grouped,) = ops_bwd.dw_bwd_grouped([(lhs.to(dev), rhs.to(dev))])
+    single = ops_bwd.dw_bwd(lhs.to(dev), rhs.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(grouped, single)
+    _close("dW, one problem, all tiles as pieces", grouped, lhs.float().T @ rhs.float())
 
 
 def test_random_shapes_every_operator_against_fp32_products():
     """Two dozen seeded random shapes through the five GEMM operators: token counts from 1 to a few
     thousand, widths that are multiples of 64 (tuned kernels: large, medium, two-launch, split and
     stream-K grids as the dispatcher picks them) or only of 8 (predicated kernel), both 16-bit
-    dtypes; each result against the fp32 product of the same rounded operands (torch's fp32 matmul
-    on the device), and the gate/up and dH epilogues against the oracle's closed forms."""
+    dtypes; each result against the fp32 product of the same rounded operands, computed on the host,
+    and the gate/up and dH epilogues against the oracle's closed forms."""
     from triton_gated_mlp.ops import bwd as ops_bwd
     from triton_gated_mlp.ops import fwd as ops_fwd
 
     dev = _dev()
     rng = np.random.default_rng(20240611)
     g = torch.Generator(device="cpu").manual_seed(99)
-    f = lambda t: t.float()
+    f = lambda t: t.float().cpu()
     for case in range(24):
         dtype = torch.float16 if case % 2 == 0 else torch.bfloat16
         unit = 8 if case % 6 == 5 else 64
@@ -921,21 +1004,20 @@ def test_random_shapes_every_operator_against_fp32_products():
         _close("U", hs.up, U)
         _close("H", hs.hidden, torch.nn.functional.silu(G) * U)
         y = ops_fwd.linear_fwd(hs.hidden, wd)
-        _close("Y", y, f(hs.hidden) @ f(wd).T, atol=ATOL * max(1.0, (N / 1024) ** 0.5))
+        _close("Y", y, f(hs.hidden) @ f(wd).T)
         # backward, from the device's own (rounded) G, U and H so that every operator is checked alone
         dg, du = ops_bwd.dh_bwd(dy, wd, hs.gate, hs.up)
-        hb = oracle.hidden_backward((f(dy) @ f(wd)).cpu(), f(hs.gate).cpu(), f(hs.up).cpu(), None, 0.0)
-        scale = max(1.0, (K / 1024) ** 0.5)
-        _close("dG", dg, hb["dG"], atol=ATOL * scale)
-        _close("dU", du, hb["dU"], atol=ATOL * scale)
+        hb = oracle.hidden_backward(f(dy) @ f(wd), f(hs.gate), f(hs.up), None, 0.0)
+        _close("dG", dg, hb["dG"])
+        _close("dU", du, hb["dU"])
         dx = ops_bwd.dx_bwd(dg, du, wg, wu)
         ref_dx = f(dg) @ f(wg) + f(du) @ f(wu)
-        _close("dX", dx, ref_dx, atol=ATOL * max(1.0, ref_dx.abs().mean().item()))
+        _close("dX", dx, ref_dx)
         pairs = [(dg, x), (du, x), (dy, hs.hidden)]
         for name, got, (a_, b_) in zip(("dW_gate", "dW_up", "dW_down"), ops_bwd.dw_bwd_grouped(pairs), pairs):
             ref = f(a_).T @ f(b_)
-            _close(name, got, ref, atol=ATOL * max(1.0, ref.abs().mean().item(), (M / 64) ** 0.5))
-        _close("dW_gate alone", ops_bwd.dw_bwd(dg, x), f(dg).T @ f(x), atol=ATOL * max(1.0, (M / 64) ** 0.5))
+            _close(name, got, ref)
+        _close("dW_gate alone", ops_bwd.dw_bwd(dg, x), f(dg).T @ f(x))
 
 
 def test_grouped_weight_gradients_equal_single_launches():
@@ -954,7 +1036,7 @@ def test_grouped_weight_gradients_equal_single_launches():
         grouped = ops_bwd.dw_bwd_grouped(pairs)
         for (a, b), got in zip(pairs, grouped):
             assert torch.equal(got, ops_bwd.dw_bwd(a, b))  # (neither form shares out tiles at these shapes)
-        _close("dW_gate grouped", grouped[0], dg.float().cpu().T @ x.float().cpu(), atol=ATOL * 40)
+        _close("dW_gate grouped", grouped[0], dg.float().cpu().T @ x.float().cpu())
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -1139,4 +1221,4 @@ def test_autocast_with_fp32_master_weights(amp_dtype):
     _close("Y", y, ref["Y"])
     names = ["dX", "dW_gate", "db_gate", "dW_up", "db_up", "dW_down", "db_down"]
     for n, g in zip(names, grads):
-        _close(n, g, ref[n], atol=ATOL * max(1.0, ref[n].abs().mean().item()))
+        _close(n, g, ref[n])

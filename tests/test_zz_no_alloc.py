@@ -17,9 +17,13 @@ def _call_pair(lib, _cabi, a, dev):
     out_ws = torch.full((C,), float("nan"), dtype=a.dtype, device=dev)
     ws = torch.empty((lib.gmlp_workspace_bytes(_cabi.GMLP_OP_COLSUM, M, 0, C, code),), dtype=torch.uint8, device=dev)
     torch.cuda.synchronize(dev)
-    before = torch.cuda.memory_allocated(dev)
+    # torch's counter only sees torch's caching allocator; free device memory as the driver reports
+    # it also moves when the library itself calls hipMalloc (gmlp_init has run: nothing is set up lazily)
+    before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
     _cabi.check(lib.gmlp_colsum_static(a.data_ptr(), out_static.data_ptr(), M, C, code, stream))
+    torch.cuda.synchronize(dev)
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before, "free device memory changed across gmlp_colsum_static"
     _cabi.check(lib.gmlp_colsum(a.data_ptr(), out_ws.data_ptr(), ws.data_ptr(), M, C, code, stream))
     torch.cuda.synchronize(dev)
     return out_static, out_ws
