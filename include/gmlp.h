@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define GMLP_ABI_VERSION 7
+#define GMLP_ABI_VERSION 8
 
 enum gmlp_dtype { GMLP_F16 = 0, GMLP_BF16 = 1, GMLP_F32 = 2 };
 
@@ -237,6 +237,45 @@ int gmlp_decode_fwd(const void* x, const void* w_gate, const void* w_up, const v
                     const void* b_gate, const void* b_up, const void* b_down, void* h_scratch,
                     void* y, void* workspace, int64_t M, int64_t K, int64_t N, int dtype, int act,
                     void* stream);
+
+/*
+ * A whole pass of the MLP in one call: validates once and enqueues every launch of the pass, so a
+ * host that drives the MLP from an interpreter pays for one foreign call per pass instead of one
+ * per GEMM (a step of a small MLP is otherwise bound by the time it takes to enqueue it).
+ *
+ * gmlp_mlp_fwd:  H = dropout(act(x·W_gateᵀ + b_gate) ⊙ (x·W_upᵀ + b_up)),  y = H·W_downᵀ + b_down
+ *   = gmlp_gateup_fwd followed by gmlp_linear_fwd, bit for bit.  Stands behind FusedGatedMLP.forward
+ *   (src/triton_gated_mlp/gated_mlp.py:230-237: FusedGatedMLPFunction.apply, then down_proj) and
+ *   mlp_hidden_states_fwd (src/triton_gated_mlp/ops/fwd.py:198-279).  h [M,N] is always written
+ *   (it is the down projection's operand); g_save, u_save [M,N] and the biases may be NULL.
+ *
+ * gmlp_mlp_bwd: every gradient of the MLP from dy [M,K]:
+ *   dG, dU (gmlp_dh_bwd) -> dx (gmlp_dx_bwd), dw_gate, dw_up, dw_down (gmlp_dw_bwd_grouped),
+ *   db_gate, db_up, db_down (gmlp_colsum_grouped), the same values as those calls give.
+ *   Stands behind mlp_hidden_states_bwd (src/triton_gated_mlp/ops/bwd.py:466-602, one host function
+ *   that enqueues the whole hidden-state backward) plus the autograd backward of down_proj.
+ *   g, u, h are what the forward pass left in g_save, u_save, h.  dg, du [M,N] are scratch the
+ *   caller provides (they hold dG and dU on return).  Any output pointer may be NULL: that gradient
+ *   is not computed, and what only it needs is not read (with dx, dw_gate, dw_up, db_gate and
+ *   db_up all NULL nothing behind dG, dU runs and w_down, g, u, dg, du may be NULL too).
+ *   Every launch goes to `stream`, in that order.
+ *
+ * workspace: gmlp_mlp_workspace_bytes(GMLP_PASS_FWD or GMLP_PASS_BWD, M, K, N, dtype) bytes (may be
+ * NULL or smaller for a pass without bias gradients: launches then take their plain form, with the
+ * same results up to the order of fp32 additions; bias gradients need it and fail with GMLP_EINVAL
+ * without).
+ */
+enum gmlp_pass { GMLP_PASS_FWD = 0, GMLP_PASS_BWD = 1 };
+size_t gmlp_mlp_workspace_bytes(int pass, int64_t M, int64_t K, int64_t N, int dtype);
+int gmlp_mlp_fwd(const void* x, const void* w_gate, const void* w_up, const void* w_down, const void* b_gate,
+                 const void* b_up, const void* b_down, void* y, void* h, void* g_save, void* u_save, int64_t M,
+                 int64_t K, int64_t N, int dtype, int act, float dropout_p, uint64_t seed, uint64_t offset,
+                 void* workspace, size_t workspace_bytes, void* stream);
+int gmlp_mlp_bwd(const void* dy, const void* x, const void* w_gate, const void* w_up, const void* w_down,
+                 const void* g, const void* u, const void* h, void* dg, void* du, void* dx, void* dw_gate,
+                 void* dw_up, void* dw_down, void* db_gate, void* db_up, void* db_down, int64_t M, int64_t K,
+                 int64_t N, int dtype, int act, float dropout_p, uint64_t seed, uint64_t offset, void* workspace,
+                 size_t workspace_bytes, void* stream);
 
 /* Writes the dropout keep mask (1 = keep) for an [M,N] tensor; the test oracle of the generator. */
 int gmlp_dropout_mask(uint8_t* mask, int64_t M, int64_t N, float dropout_p, uint64_t seed,

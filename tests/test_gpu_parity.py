@@ -974,6 +974,64 @@ def test_grouped_launch_of_one_problem_whose_tiles_all_go_to_streamk():
     _close("dW, one problem, all tiles as pieces", grouped, lhs.float().T @ rhs.float())
 
 
+@pytest.mark.parametrize(
+    "M,K,N,dtype,bias,p",
+    [
+        (2048, 2048, 5632, torch.bfloat16, True, 0.1),   # mid-size grids, biases, dropout
+        (300, 1024, 4096, torch.float16, True, 0.0),     # short batch: split reductions, ragged rows
+        (2048, 4352, 5120, torch.float16, False, 0.25),  # stream-K in the forward GEMMs
+        (1000, 520, 1048, torch.bfloat16, True, 0.0),    # widths that are multiples of 8 only (predicated kernels)
+        (192, 512, 768, torch.float32, True, 0.1),       # float32 path
+    ],
+)
+def test_whole_pass_entry_points_equal_the_separate_launches(M, K, N, dtype, bias, p):
+    """gmlp_mlp_fwd and gmlp_mlp_bwd (one library call per pass; what the module uses) give, bit for
+    bit, what the per-GEMM entry points give when called one after the other, call after call, and
+    leave out exactly the gradients that were not asked for.  (The separate entry
+    points are the ones held against the oracle throughout this file; the module-level cases go
+    through the one-call entries and are held against the oracle as well.)"""
+    from triton_gated_mlp.ops import bwd as ops_bwd
+    from triton_gated_mlp.ops import fwd as ops_fwd
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(31)
+    rnd = lambda *shape, s=1.0: (s * torch.randn(*shape, generator=g)).to(dtype).to(dev)
+    x, wg, wu, wd, dy = rnd(M, K), rnd(N, K, s=0.03), rnd(N, K, s=0.03), rnd(K, N, s=0.03), rnd(M, K)
+    bg, bu, bd = (rnd(N, s=0.1), rnd(N, s=0.1), rnd(K, s=0.1)) if bias else (None, None, None)
+    seed, off = 77, 2
+    hs = ops_fwd.gateup_fwd(x, wg, bg, wu, bu, p, seed, off, save_activations=True)
+    y_ref = ops_fwd.linear_fwd(hs.hidden, wd, bd)
+    y, hs1 = ops_fwd.mlp_fwd(x, wg, bg, wu, bu, wd, bd, p, seed, off, save_activations=True)
+    assert torch.equal(y, y_ref) and torch.equal(hs1.hidden, hs.hidden)
+    assert torch.equal(hs1.gate, hs.gate) and torch.equal(hs1.up, hs.up)
+    y2, hs2 = ops_fwd.mlp_fwd(x, wg, bg, wu, bu, wd, bd, p, seed, off, save_activations=False)
+    assert torch.equal(y2, y_ref) and hs2.gate is None and hs2.up is None
+
+    dg, du = ops_bwd.dh_bwd(dy, wd, hs.gate, hs.up, p, seed, off)
+    ref = {
+        "dx": ops_bwd.dx_bwd(dg, du, wg, wu),
+        "dW_gate": None, "db_gate": None, "dW_up": None, "db_up": None, "dW_down": None, "db_down": None,
+    }
+    ref["dW_gate"], ref["dW_up"], ref["dW_down"] = ops_bwd.dw_bwd_grouped([(dg, x), (du, x), (dy, hs.hidden)])
+    if bias:
+        ref["db_gate"], ref["db_up"], ref["db_down"] = ops_bwd.colsum_grouped([dg, du, dy])
+    names = list(ref)
+    all_of = tuple(ref[n] is not None for n in names)
+    for call in range(2):
+        got = ops_bwd.mlp_bwd(dy, x, wg, wu, wd, hs.gate, hs.up, hs.hidden, all_of, p, seed, off)
+        torch.cuda.synchronize()
+        for n, a, b in zip(names, got, (ref[n] for n in names)):
+            assert (a is None) == (b is None), n
+            assert a is None or torch.equal(a, b), f"{n} differs (call {call})"
+    # subsets: only the input gradient; only the down projection's gradients; everything but dX
+    for want in ((True,) + (False,) * 6, (False,) * 5 + (True, bias), (False,) + all_of[1:]):
+        got = ops_bwd.mlp_bwd(dy, x, wg, wu, wd, hs.gate, hs.up, hs.hidden, want, p, seed, off)
+        torch.cuda.synchronize()
+        for n, w, a in zip(names, want, got):
+            assert (a is not None) == bool(w), n
+            assert a is None or torch.equal(a, ref[n]), f"{n} differs for subset {want}"
+
+
 def test_random_shapes_every_operator_against_fp32_products():
     """Two dozen seeded random shapes through the five GEMM operators: token counts from 1 to a few
     thousand, widths that are multiples of 64 (tuned kernels: large, medium, two-launch, split and

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"libgmlp.so does not export {name}"
     assert sorted(_cabi.EXPORTED_SYMBOLS) == declared, "ctypes signature table and gmlp.h disagree"
-    assert lib.gmlp_abi_version() == 7
+    assert lib.gmlp_abi_version() == 8
 
 
 def _buf(nbytes=4096):
@@ -101,6 +101,59 @@ def test_argument_validation_returns_codes_without_touching_the_device():
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DH_BWD, 2048, 2048, 5632, 1) == 0  # short reduction: not worth it
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DW_BWD_GROUPED, 0, 0, 0, 0) == 512 * 65536 * 4
     assert lib.gmlp_workspace_bytes(_cabi.GMLP_OP_DW_BWD_GROUPED, 0, 0, 0, 2) == 0
+
+
+def test_whole_pass_entry_points_validate_before_touching_the_device():
+    """gmlp_mlp_fwd / gmlp_mlp_bwd: one call per pass.  Their own argument checks (and the workspace
+    plan) run on the host before anything is enqueued."""
+    lib = _cabi.lib()
+    _, a = _buf()
+    err = lambda: lib.gmlp_last_error().decode()
+    fwd = lambda *ptrs, M=8, K=8, N=8, dt=0, act=0, p=0.0: lib.gmlp_mlp_fwd(*ptrs, M, K, N, dt, act, p, 0, 0, None, 0, None)
+    full = (a, a, a, a, None, None, None, a, a, None, None)  # x, wg, wu, wd, biases, y, h, g_save, u_save
+    for missing in (0, 1, 2, 3, 7, 8):  # x, the three weights, y, h
+        ptrs = list(full)
+        ptrs[missing] = None
+        assert fwd(*ptrs) == -1 and "NULL" in err() and "gmlp_mlp_fwd" in err()
+    assert fwd(*full, dt=5) == -1 and "dtype" in err()
+    assert fwd(*full, act=9) == -1 and "act" in err()
+    assert fwd(*full, p=1.0) == -1
+    assert fwd(*full, K=12) == -2 and "multiple of 8" in err()
+    assert fwd(*full, M=0) == -2
+    misaligned = list(full)
+    misaligned[4] = a + 2  # b_gate
+    assert fwd(*misaligned) == -3 and "b_gate" in err()
+
+    def bwd(dy=a, x=a, wg=a, wu=a, wd=a, g=a, u=a, h=a, dg=a, du=a, dx=a, dwg=a, dwu=a, dwd=a, dbg=None, dbu=None,
+            dbd=None, M=8, K=8, N=8, dt=0, act=0, p=0.0, ws=None, nws=0):
+        return lib.gmlp_mlp_bwd(dy, x, wg, wu, wd, g, u, h, dg, du, dx, dwg, dwu, dwd, dbg, dbu, dbd, M, K, N, dt, act, p,
+                                0, 0, ws, nws, None)
+
+    assert bwd(dy=None) == -1 and "'dy'" in err() and "gmlp_mlp_bwd" in err()
+    # what a requested output needs must be there ...
+    assert bwd(g=None) == -1 and "'g'" in err()
+    assert bwd(dg=None) == -1 and "'dg'" in err()
+    assert bwd(wd=None) == -1 and "'w_down'" in err()
+    assert bwd(x=None) == -1 and "'x'" in err()
+    assert bwd(h=None) == -1 and "'h'" in err()
+    assert bwd(wg=None) == -1 and "'w_gate'" in err()
+    # ... bad codes and shapes are refused like everywhere else
+    assert bwd(dt=3) == -1 and bwd(act=-1) == -1 and bwd(p=float("nan")) == -1
+    assert bwd(N=20) == -2 and bwd(M=0) == -2
+    assert bwd(dx=a + 4) == -3 and "'dx'" in err()
+    # bias gradients need the workspace (their partial sums live there); the others do without
+    assert bwd(dbg=a) == -1 and "workspace" in err()
+    # workspace plan: forward = the larger of its two launches; backward = three regions that do not alias
+    q = lib.gmlp_workspace_bytes
+    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_FWD, 64, 8192, 28672, 0) == max(
+        q(_cabi.GMLP_OP_GATEUP_FWD, 64, 8192, 28672, 0), q(_cabi.GMLP_OP_LINEAR_FWD, 64, 28672, 8192, 0)) > 0
+    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_FWD, 8192, 4096, 14336, 0) == 0
+    cs = lambda M, C: q(_cabi.GMLP_OP_COLSUM, M, 0, C, 0)
+    M, K, N = 8192, 4096, 14336  # nothing for dH / dX, stream-K for the grouped weight gradients, column sums
+    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, 0) == 384 * 65536 * 4 + 2 * cs(M, N) + cs(M, K)
+    M, K, N = 300, 4096, 14336  # a short batch: split reduction for dX
+    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, 1) >= q(_cabi.GMLP_OP_DX_BWD, M, K, N, 1) > 0
+    assert lib.gmlp_mlp_workspace_bytes(7, 8, 8, 8, 0) == 0 and lib.gmlp_mlp_workspace_bytes(0, 0, 8, 8, 0) == 0
 
 
 def test_error_codes_map_to_python_exceptions():

@@ -17,7 +17,8 @@ from torch import Tensor
 GMLP_F16, GMLP_BF16, GMLP_F32 = 0, 1, 2
 GMLP_OP_DECODE_FWD, GMLP_OP_COLSUM, GMLP_OP_LINEAR_FWD, GMLP_OP_DX_BWD, GMLP_OP_GATEUP_FWD = 0, 1, 2, 3, 4
 GMLP_OP_DH_BWD, GMLP_OP_DW_BWD, GMLP_OP_DW_BWD_GROUPED = 5, 6, 7
-ABI_VERSION = 7
+ABI_VERSION = 8
+GMLP_PASS_FWD, GMLP_PASS_BWD = 0, 1
 
 # hidden_act name -> GMLP_ACT_* code.  The names are those of the reference's ACT2CLS / ACT_FWD
 # tables (src/triton_gated_mlp/gated_mlp.py:17-37).
@@ -67,6 +68,15 @@ _SIGNATURES = {
     "gmlp_colsum_grouped": (_int, [_int, _c_ptr, _c_ptr, _c_ptr, _i64, _c_ptr, _int, _c_ptr]),
     "gmlp_decode_fwd": (_int, [_c_ptr] * 10 + [_i64, _i64, _i64, _int, _int, _c_ptr]),
     "gmlp_dropout_mask": (_int, [_c_ptr, _i64, _i64, _f32, _u64, _u64, _c_ptr]),
+    "gmlp_mlp_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _i64, _i64, _int]),
+    "gmlp_mlp_fwd": (
+        _int,
+        [_c_ptr] * 11 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr, ctypes.c_size_t, _c_ptr],
+    ),
+    "gmlp_mlp_bwd": (
+        _int,
+        [_c_ptr] * 17 + [_i64, _i64, _i64, _int, _int, _f32, _u64, _u64, _c_ptr, ctypes.c_size_t, _c_ptr],
+    ),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -163,3 +173,17 @@ def ptr(t: Optional[Tensor]) -> Optional[int]:
 
 def stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+_MLP_WS = {}
+
+
+def mlp_workspace_bytes(which: int, M: int, K: int, N: int, code: int, device: torch.device) -> int:
+    """gmlp_mlp_workspace_bytes, remembered per problem and device (the plan depends on the device's
+    compute-unit count; call with `device` current)."""
+    key = (which, M, K, N, code, device.index)
+    n = _MLP_WS.get(key)
+    if n is None:
+        n = _MLP_WS[key] = lib().gmlp_mlp_workspace_bytes(which, M, K, N, code)
+    return n
+

@@ -150,10 +150,10 @@ class FusedGatedMLPFullFunction(Function):
     ):
         needs_grad = any(ctx.needs_input_grad[:7])
         keep = needs_grad and not recompute
-        hs = _fwd.gateup_fwd(
-            x, W_gate, b_gate, W_up, b_up, dropout_p, seed, offset, save_activations=keep, act_fn=act_fn
+        # one library call enqueues the whole pass
+        y, hs = _fwd.mlp_fwd(
+            x, W_gate, b_gate, W_up, b_up, W_down, b_down, dropout_p, seed, offset, save_activations=keep, act_fn=act_fn
         )
-        y = _fwd.linear_fwd(hs.hidden, W_down, b_down)
         if keep:
             ctx.save_for_backward(x, W_gate, W_up, W_down, hs.gate, hs.up, hs.hidden)
         elif needs_grad:
@@ -178,33 +178,12 @@ class FusedGatedMLPFullFunction(Function):
         else:
             x, W_gate, W_up, W_down, gate, up, hidden = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dy = dy.contiguous()
-        dx = dW_gate = db_gate = dW_up = db_up = dW_down = db_down = None
-        dw_jobs = []  # (slot, lhs, rhs): the weight gradients go out as one grouped launch
-        db_jobs = []  # (slot, array): so do the bias gradients
-        if any(need[:5]):
-            dg, du = _bwd.dh_bwd(dy, W_down, gate, up, p, seed, offset, ctx.act_fn)
-            if need[0]:
-                dx = _bwd.dx_bwd(dg, du, W_gate, W_up)
-            if need[1]:
-                dw_jobs.append(("gate", dg, x))
-            if ctx.has_bias[0] and need[2]:
-                db_jobs.append(("gate", dg))
-            if need[3]:
-                dw_jobs.append(("up", du, x))
-            if ctx.has_bias[1] and need[4]:
-                db_jobs.append(("up", du))
-        if need[5]:
-            dw_jobs.append(("down", dy, hidden))
-        if ctx.has_bias[2] and need[6]:
-            db_jobs.append(("down", dy))
-        if dw_jobs:
-            grads = dict(zip([j[0] for j in dw_jobs], _bwd.dw_bwd_grouped([(j[1], j[2]) for j in dw_jobs])))
-            dW_gate, dW_up, dW_down = grads.get("gate"), grads.get("up"), grads.get("down")
-        if db_jobs:
-            grads = dict(zip([j[0] for j in db_jobs], _bwd.colsum_grouped([j[1] for j in db_jobs])))
-            db_gate, db_up, db_down = grads.get("gate"), grads.get("up"), grads.get("down")
-        return dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down, None, None, None, None, None
+        has = ctx.has_bias
+        want = (need[0], need[1], has[0] and need[2], need[3], has[1] and need[4], need[5], has[2] and need[6])
+        # one library call enqueues the whole pass: dH with the gating epilogue, dX, the three
+        # weight gradients as one grid, the bias gradients as one pair of launches
+        grads = _bwd.mlp_bwd(dy, x, W_gate, W_up, W_down, gate, up, hidden, want, p, seed, offset, ctx.act_fn)
+        return grads + (None, None, None, None, None)
 
 
 class FusedGatedMLP(_GatedMLPBase):
@@ -287,8 +266,7 @@ class FusedGatedMLP(_GatedMLPBase):
             # short batch's kernels take to enqueue), and the weight-streaming kernels for skinny M.
             if _fwd.decode_preferred(M, K, self.intermediate_size, x2.dtype, _compute_units(x2.device)):
                 return _fwd.decode_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, self.act_fn)
-            hs = _fwd.gateup_fwd(x2, W_gate, b_gate, W_up, b_up, 0.0, 0, 0, save_activations=False, act_fn=self.act_fn)
-            return _fwd.linear_fwd(hs.hidden, W_down, b_down)
+            return _fwd.mlp_fwd(x2, W_gate, b_gate, W_up, b_up, W_down, b_down, act_fn=self.act_fn)[0]
         if x2.is_cuda and torch.cuda.is_current_stream_capturing():
             # Capturing forward + backward with torch.cuda.graph has ended in a host-side crash inside
             # the runtime's end-of-capture call on ROCm 7.2; until its cause is known the module

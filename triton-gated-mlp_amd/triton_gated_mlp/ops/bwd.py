@@ -243,6 +243,60 @@ def colsum_grouped(arrays):
     return outs
 
 
+def mlp_bwd(
+    dy: Tensor,
+    x: Tensor,
+    W_gate: Tensor,
+    W_up: Tensor,
+    W_down: Tensor,
+    g: Tensor,
+    u: Tensor,
+    h: Tensor,
+    need=(True,) * 7,
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    act_fn: str = "silu",
+):
+    """Whole backward pass in one library call (gmlp_mlp_bwd).
+
+    `need` = which of (dx, dW_gate, db_gate, dW_up, db_up, dW_down, db_down) to compute; returns
+    that 7-tuple with None for the others.  dG, dU and the library's workspace share one scratch
+    allocation that is dropped on return."""
+    M, K = dy.shape
+    N = W_down.shape[1]
+    if (
+        tuple(x.shape) != (M, K) or tuple(W_gate.shape) != (N, K) or tuple(W_up.shape) != (N, K)
+        or tuple(W_down.shape) != (K, N) or tuple(g.shape) != (M, N) or tuple(u.shape) != (M, N)
+        or tuple(h.shape) != (M, N)
+    ):
+        raise ValueError("dimension mismatch among dy, x, the weights and the kept activations")
+    dev = _cabi.require_gpu(dy, x, W_gate, W_up, W_down, g, u, h)
+    code = _cabi.dtype_code(dy.dtype)
+    act = _cabi.act_code(act_fn)
+    dy, x, W_gate, W_up, W_down, g, u, h = (_c(t) for t in (dy, x, W_gate, W_up, W_down, g, u, h))
+    shapes = ((M, K), (N, K), (N,), (N, K), (N,), (K, N), (K,))
+    if M == 0:
+        return tuple(torch.zeros(s, dtype=dy.dtype, device=dev) if n else None for s, n in zip(shapes, need))
+    outs = [torch.empty(s, dtype=dy.dtype, device=dev) if n else None for s, n in zip(shapes, need)]
+    dx, dwg, dbg, dwu, dbu, dwd, dbd = outs
+    with torch.cuda.device(dev):
+        nbytes = _cabi.mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, code, dev)
+        plane = (M * N * dy.element_size() + 255) // 256 * 256
+        arena = torch.empty((2 * plane + nbytes,), dtype=torch.uint8, device=dev)
+        base = arena.data_ptr()
+        _cabi.check(
+            _cabi.lib().gmlp_mlp_bwd(
+                _cabi.ptr(dy), _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(W_down),
+                _cabi.ptr(g), _cabi.ptr(u), _cabi.ptr(h), base, base + plane,
+                _cabi.ptr(dx), _cabi.ptr(dwg), _cabi.ptr(dwu), _cabi.ptr(dwd), _cabi.ptr(dbg), _cabi.ptr(dbu),
+                _cabi.ptr(dbd), M, K, N, code, act, float(dropout_p), int(seed), int(offset),
+                base + 2 * plane if nbytes else None, nbytes, _cabi.stream_ptr(dev),
+            )
+        )
+    return tuple(outs)
+
+
 def mlp_hidden_states_bwd(
     x: Tensor,
     W_up: Tensor,

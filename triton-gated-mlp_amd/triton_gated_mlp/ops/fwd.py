@@ -127,6 +127,57 @@ def linear_fwd(a: Tensor, W: Tensor, bias: Optional[Tensor] = None) -> Tensor:
     return out
 
 
+def mlp_fwd(
+    x: Tensor,
+    W_gate: Tensor,
+    b_gate: Optional[Tensor],
+    W_up: Tensor,
+    b_up: Optional[Tensor],
+    W_down: Tensor,
+    b_down: Optional[Tensor],
+    dropout_p: float = 0.0,
+    seed: int = 0,
+    offset: int = 0,
+    save_activations: bool = False,
+    act_fn: str = "silu",
+):
+    """Whole forward pass in one library call (gmlp_mlp_fwd): returns (y, HiddenStates).
+
+    The same kernels as gateup_fwd followed by linear_fwd, enqueued by one foreign call; G, U and H
+    share one allocation when they are kept for the backward pass."""
+    validate_dimensions(x, W_up, b_up, W_gate, b_gate)
+    M, K = x.shape
+    N = W_up.shape[0]
+    if tuple(W_down.shape) != (K, N):
+        raise ValueError(f"dimension mismatch in W_down {tuple(W_down.shape)}")
+    if b_down is not None and tuple(b_down.shape) != (K,):
+        raise ValueError("dimension mismatch in b_down")
+    act = _cabi.act_code(act_fn)
+    dev = _cabi.require_gpu(x, W_gate, b_gate, W_up, b_up, W_down, b_down)
+    code = _cabi.dtype_code(x.dtype)
+    x, W_gate, W_up, W_down = _c(x), _c(W_gate), _c(W_up), _c(W_down)
+    b_gate, b_up, b_down = _c(b_gate), _c(b_up), _c(b_down)
+    y = torch.empty((M, K), dtype=x.dtype, device=dev)
+    if save_activations:
+        g, u, h = torch.empty((3, M, N), dtype=x.dtype, device=dev).unbind(0)
+    else:
+        g = u = None
+        h = torch.empty((M, N), dtype=x.dtype, device=dev)
+    if M > 0:
+        with torch.cuda.device(dev):
+            nbytes = _cabi.mlp_workspace_bytes(_cabi.GMLP_PASS_FWD, M, K, N, code, dev)
+            ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
+            _cabi.check(
+                _cabi.lib().gmlp_mlp_fwd(
+                    _cabi.ptr(x), _cabi.ptr(W_gate), _cabi.ptr(W_up), _cabi.ptr(W_down), _cabi.ptr(b_gate),
+                    _cabi.ptr(b_up), _cabi.ptr(b_down), _cabi.ptr(y), _cabi.ptr(h), _cabi.ptr(g), _cabi.ptr(u),
+                    M, K, N, code, act, float(dropout_p), int(seed), int(offset),
+                    _cabi.ptr(ws), nbytes, _cabi.stream_ptr(dev),
+                )
+            )
+    return y, HiddenStates(h, g, u, None)
+
+
 DECODE_MAX_M = 32
 DECODE_PREFERRED_MAX_M = 32
 
