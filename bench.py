@@ -42,15 +42,30 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
 M, K, N = 8192, 4096, 14336
 DTYPE = torch.float16
-# HBM-side bytes per grouped weight-gradient launch (its three kernels together), from two
-# `rocprofv3 --pmc` runs, FETCH_SIZE x 2.0 (what the counter reads for a plain copy of known size)
-# + WRITE_SIZE x 1.0: profiles/gemm_hbm_traffic_fp16_M8192_K4096_N14336.txt.  To be re-measured
-# whenever the weight-gradient kernels or their tile order change.
-DW_GROUP_TRAFFIC_BYTES = 5.22e9
 DW_GROUP_ALGORITHMIC_BYTES = 1.258e9  # dG, dU, dY, H once, x twice, three dW once
-# The same for one skinny-M forward at M=16, K=8192, N=28672 (both kernels):
-# profiles/decode_hbm_traffic_fp16_M16_K8192_N28672.txt.
-DECODE_TRAFFIC_BYTES = 1.469e9
+# HBM-side bytes per call (`roofline.traffic`) are not measured by this script: they come from two
+# `rocprofv3 --pmc` runs of it (FETCH_SIZE, WRITE_SIZE), summarised in the files below, each of
+# which carries one line `traffic_bytes_per_call = <bytes>`.  The JSON line names the file and its
+# git blob hash next to the figure, so a figure that predates a kernel change shows.
+DW_GROUP_TRAFFIC_PROFILE = "profiles/gemm_hbm_traffic_fp16_M8192_K4096_N14336.txt"
+DECODE_TRAFFIC_PROFILE = "profiles/decode_hbm_traffic_fp16_M16_K8192_N28672.txt"
+
+
+def _traffic_from_profile(rel):
+    """(bytes per call or None, provenance) from a committed rocprofv3 summary."""
+    import hashlib
+    import re
+
+    path = ROOT / rel
+    try:
+        raw = path.read_bytes()
+    except OSError:
+        return None, {"file": rel, "error": "missing"}
+    m = re.search(rb"^traffic_bytes_per_call\s*=\s*([0-9.eE+]+)", raw, flags=re.M)
+    blob = hashlib.sha1(b"blob %d\0" % len(raw) + raw).hexdigest()
+    note = "HBM-side bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0), factors from a plain 256 MiB copy"
+    return (float(m.group(1)) if m else None), {"file": rel, "git_blob": blob, "how": note}
+
 
 _flush_buf = None
 
@@ -105,18 +120,27 @@ def _r(x, n=4):
     return round(x, n)
 
 
+def _stated_inputs(mod, m, k, dev, dt, backward, seed=0):
+    """Fills a gated-MLP module and makes its inputs from the distributions the baseline
+    configurations state: weights ~ N(0, 0.02), biases ~ U(-0.01, 0.01), x ~ N(0, 1), upstream
+    gradient ~ N(0, 1); seeded, generated on the device in fp32 and rounded to `dt`.  (Operand
+    statistics matter to the timing: the chip runs these kernels at its power cap.)"""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    with torch.no_grad():
+        for lin in (mod.gate_proj, mod.up_proj, mod.down_proj):
+            lin.weight.copy_(torch.empty(lin.weight.shape, device=dev).normal_(0.0, 0.02, generator=g))
+            if lin.bias is not None:
+                lin.bias.copy_(torch.empty(lin.bias.shape, device=dev).uniform_(-0.01, 0.01, generator=g))
+    x = torch.empty(m, k, device=dev).normal_(0.0, 1.0, generator=g).to(dt).requires_grad_(backward)
+    dy = torch.empty(m, k, device=dev).normal_(0.0, 1.0, generator=g).to(dt)
+    return x, dy
+
+
 def _make_module(dev):
     from triton_gated_mlp import FusedGatedMLP
 
-    g = torch.Generator().manual_seed(0)
-    mlp = FusedGatedMLP(hidden_size=K, intermediate_size=N, bias=False, dropout_p=0.0)
-    with torch.no_grad():
-        mlp.gate_proj.weight.copy_(0.02 * torch.randn(N, K, generator=g))
-        mlp.up_proj.weight.copy_(0.02 * torch.randn(N, K, generator=g))
-        mlp.down_proj.weight.copy_(0.02 * torch.randn(K, N, generator=g))
-    mlp = mlp.to(dev).to(DTYPE)
-    x = torch.randn(M, K, generator=g).to(DTYPE).to(dev).requires_grad_(True)
-    dY = torch.randn(M, K, generator=g).to(DTYPE).to(dev)
+    mlp = FusedGatedMLP(hidden_size=K, intermediate_size=N, bias=False, dropout_p=0.0).to(dev).to(DTYPE)
+    x, dY = _stated_inputs(mlp, M, K, dev, DTYPE, True)
     return mlp, x, dY
 
 
@@ -230,8 +254,7 @@ def _config_lines(dev):
         mlp = FusedGatedMLP(hidden_size=k, intermediate_size=n, bias=bias, dropout_p=p).to(dev).to(dt)
         mlp.train(bwd)
         mlp.dropout_seed = 1234
-        x = torch.randn(m, k, device=dev, dtype=dt, requires_grad=bwd)
-        dy = torch.randn(m, k, device=dev, dtype=dt)
+        x, dy = _stated_inputs(mlp, m, k, dev, dt, bwd)
         params = list(mlp.parameters())
 
         def step():
@@ -264,6 +287,7 @@ def _config_lines(dev):
     Wu = torch.empty(n, k, dtype=torch.float16, device=dev).normal_(0, 0.02)
     Wd = torch.empty(k, n, dtype=torch.float16, device=dev).normal_(0, 0.02)
     nbytes = 3 * k * n * 2 + m * k * 2 + 2 * m * n * 2 + m * k * 2
+    traffic, traffic_src = _traffic_from_profile(DECODE_TRAFFIC_PROFILE)
     t = _bench(lambda: F.decode_fwd(x, Wg, None, Wu, None, Wd, None), rep_ms=30.0, min_reps=20)
     # CPU: one sixteenth of the intermediate width (the CPU is bound by reading the weights as well)
     cpu_n = n // 16
@@ -273,9 +297,8 @@ def _config_lines(dev):
                 "bytes": nbytes, "gbps": _r(nbytes / t["p50"] / 1e6, 1), "tflops": _r(6.0 * m * n * k / t["p50"] / 1e9, 1),
                 "cache_flush_between_reps": True,
                 "roofline": {"bound": "hbm", "achieved": _r(nbytes / t["p50"] / 1e6, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                             "frac": _r(nbytes / t["p50"] / 1e6 / PEAK_HBM_GBPS), "traffic": DECODE_TRAFFIC_BYTES,
-                             "traffic_note": "HBM-side bytes per forward from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
-                                             "(profiles/decode_hbm_traffic_fp16_M16_K8192_N28672.txt)"}},
+                             "frac": _r(nbytes / t["p50"] / 1e6 / PEAK_HBM_GBPS), "traffic": traffic,
+                             "traffic_source": traffic_src}},
         "cpu": {"ms": _r(cpu_t * 1e3, 1), "gbps": _r(3 * k * cpu_n * 4 / cpu_t / 1e9, 1), "tflops": _r(cpu_tf, 4),
                 "sample": f"all 16 rows, intermediate columns 0..{cpu_n - 1} of {n} (fp32 weights: {3 * k * cpu_n * 4 / 1e6:.0f} MB), "
                           "fp32 torch-CPU oracle, median of 2 after 1 warm-up"},
@@ -290,7 +313,7 @@ def _edge_shapes(dev):
     (forward; the down projection splits its reduction), a batch of one and a half rounds of tiles
     (stream-K) and a batch whose 2.3 GB activations are beyond 32-bit byte offsets (fwd+bwd; the
     module runs it as two row chunks)."""
-    from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP
+    from triton_gated_mlp import EagerGatedMLP, FusedGatedMLP, copy_weights
 
     out = {}
     for name, (m, k, n, bwd) in {
@@ -301,8 +324,8 @@ def _edge_shapes(dev):
     }.items():
         fused = FusedGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
         eager = EagerGatedMLP(hidden_size=k, intermediate_size=n, bias=False).to(dev).to(DTYPE)
-        x = torch.randn(m, k, device=dev, dtype=DTYPE, requires_grad=bwd)
-        dy = torch.randn(m, k, device=dev, dtype=DTYPE)
+        x, dy = _stated_inputs(fused, m, k, dev, DTYPE, bwd)
+        copy_weights(fused, eager)
         res = {}
         for label, mod in (("ms", fused), ("torch_eager_ms", eager)):
             params = list(mod.parameters())
@@ -345,6 +368,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip per-kernel breakdown, other configurations and edge shapes")
+    ap.add_argument("--step-only", action="store_true",
+                    help="time the steps and nothing else (no roofline launch, quantiles, extras or CPU leg): what a kernel "
+                         "trace of the step itself is taken from")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -384,6 +410,12 @@ def main():
     flop_step = 18.0 * M * N * K
     tflops = flop_step / (ms_per_step * 1e-3) / 1e12
 
+    if args.step_only:
+        print(json.dumps({"metric": "fwd+bwd TFLOP/s & % MFMA peak, fp16 M=8192 K=4096 N=14336 (1 GPU)", "value": round(tflops, 2),
+                          "unit": "TFLOP/s", "ms_per_step": round(ms_per_step, 4), "steps": args.steps, "warmup": args.warmup,
+                          "note": "--step-only: the timed steps alone"}), flush=True)
+        return
+
     # dominant launch: dW_gate, dW_up and dW_down through gmlp_dw_bwd_grouped (6*M*N*K FLOP): one grid
     # of whole rounds of tiles, the pieces of the last half round's tiles (stream-K) and their sums;
     # events on the launch stream around the three kernels
@@ -394,17 +426,21 @@ def main():
     xd = x.detach()
     hs = F.gateup_fwd(xd, Wg, None, Wu, None, save_activations=True)
     dg, du = B.dh_bwd(dY, Wd, hs.gate, hs.up)
-    t = _bench(lambda: B.dw_bwd_grouped([(dg, xd), (du, xd), (dY, hs.hidden)]), rep_ms=60.0, min_reps=max(args.steps, 10), flush=False)
+    dw_call = lambda: B.dw_bwd_grouped([(dg, xd), (du, xd), (dY, hs.hidden)])
+    # back to back (as the kernels run under rocprofv3 in profiles/) and behind a cache flush (as the
+    # `kernels` block times every launch); inside a step the call sits between the two
+    t = _bench(dw_call, rep_ms=60.0, min_reps=max(args.steps, 10), flush=False)
+    t_flushed = _bench(dw_call, rep_ms=40.0, min_reps=10, flush=True)
     del dg, du, hs
     dom_flop = 6.0 * M * N * K
+    traffic, traffic_src = _traffic_from_profile(DW_GROUP_TRAFFIC_PROFILE)
     roofline = dict(
         _mfma_block(dom_flop, t["mean"]),
         kernel="gmlp_dw_bwd_grouped (dW_gate + dW_up + dW_down): gemm_group_kernel_pipelined<f16,256,256,16,...,EpiStore> over 2560 "
                "tiles, gemm_kernel_pipelined<...,stream-K> over the pieces of the other 128, streamk_fixup_kernel",
-        avg_launch_ms=_r(t["mean"]), p50_launch_ms=_r(t["p50"]), flop_per_launch=dom_flop, traffic=DW_GROUP_TRAFFIC_BYTES,
-        algorithmic_bytes=DW_GROUP_ALGORITHMIC_BYTES,
-        traffic_note="HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
-                     "(profiles/gemm_hbm_traffic_fp16_M8192_K4096_N14336.txt)",
+        avg_launch_ms=_r(t["mean"]), p50_launch_ms=_r(t["p50"]), launches_timed=t["reps"], timing="HIP events on the launch stream, "
+        "calls back to back, no cache flush", flushed_launch_ms=_r(t_flushed["mean"]), frac_flushed=_r(dom_flop / t_flushed["mean"] / 1e9 / PEAK_MFMA_F16_TFLOPS),
+        flop_per_launch=dom_flop, traffic=traffic, algorithmic_bytes=DW_GROUP_ALGORITHMIC_BYTES, traffic_source=traffic_src,
     )
 
     line = {
