@@ -143,14 +143,14 @@ def test_whole_pass_entry_points_validate_before_touching_the_device():
     assert bwd(dx=a + 4) == -3 and "'dx'" in err()
     # bias gradients need the workspace (their partial sums live there); the others do without
     assert bwd(dbg=a) == -1 and "workspace" in err()
-    # workspace plan: forward = the larger of its two launches; backward = three regions that do not alias
+    # workspace plan: forward = the larger of its two launches; backward = the largest of its launches' requests
     q = lib.gmlp_workspace_bytes
     assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_FWD, 64, 8192, 28672, 0) == max(
         q(_cabi.GMLP_OP_GATEUP_FWD, 64, 8192, 28672, 0), q(_cabi.GMLP_OP_LINEAR_FWD, 64, 28672, 8192, 0)) > 0
     assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_FWD, 8192, 4096, 14336, 0) == 0
     cs = lambda M, C: q(_cabi.GMLP_OP_COLSUM, M, 0, C, 0)
     M, K, N = 8192, 4096, 14336  # nothing for dH / dX, stream-K for the grouped weight gradients, column sums
-    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, 0) == 384 * 65536 * 4 + 2 * cs(M, N) + cs(M, K)
+    assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, 0) == max(384 * 65536 * 4, 2 * cs(M, N) + cs(M, K))
     M, K, N = 300, 4096, 14336  # a short batch: split reduction for dX
     assert lib.gmlp_mlp_workspace_bytes(_cabi.GMLP_PASS_BWD, M, K, N, 1) >= q(_cabi.GMLP_OP_DX_BWD, M, K, N, 1) > 0
     assert lib.gmlp_mlp_workspace_bytes(7, 8, 8, 8, 0) == 0 and lib.gmlp_mlp_workspace_bytes(0, 0, 8, 8, 0) == 0

@@ -3,6 +3,7 @@
 // so the error paths can be exercised on a machine without a GPU.
 #include "gmlp.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdarg>
@@ -798,15 +799,13 @@ int gmlp_dropout_mask(uint8_t* mask, int64_t M, int64_t N, float dropout_p, uint
 // ---------------------------------------------------------------- whole passes in one call
 namespace {
 
-size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
-
-// Workspace of a backward pass: three regions that do not alias (the launches that use them are
-// enqueued one after the other today, but nothing in the layout relies on that).
+// Workspace of a backward pass: what its launches ask for, one after the other on one stream, so
+// one buffer of the largest request serves them all.
 struct BwdWorkspace {
   size_t act = 0;     // gmlp_dh_bwd, then gmlp_dx_bwd
   size_t dw = 0;      // gmlp_dw_bwd_grouped
   size_t colsum = 0;  // gmlp_colsum_grouped
-  size_t total() const { return align256(act) + align256(dw) + align256(colsum); }
+  size_t total() const { return std::max(act, std::max(dw, colsum)); }
 };
 BwdWorkspace plan_bwd_workspace(int64_t M, int64_t K, int64_t N, int dtype, bool gate, bool up, bool down,
                                 bool bias_gate, bool bias_up, bool bias_down) {
@@ -899,27 +898,16 @@ int gmlp_mlp_bwd(const void* dy, const void* x, const void* w_gate, const void* 
   GMLP_REQUIRE_ALIGNED(db_down); GMLP_REQUIRE_ALIGNED(workspace);
 
   const BwdWorkspace need = plan_bwd_workspace(M, K, N, dtype, dw_gate, dw_up, dw_down, db_gate, db_up, db_down);
-  // Regions in the caller's buffer; one that does not fit is left out and its launches take their
-  // plain form (same results, no split reduction or stream-K).  Bias gradients cannot do without.
-  char* base = (char*)workspace;
-  size_t left = base ? workspace_bytes : 0;
-  auto carve = [&](size_t bytes, void** ptr, size_t* got) {
-    *ptr = nullptr;
-    *got = 0;
-    if (bytes == 0 || align256(bytes) > left) return;
-    *ptr = base;
-    *got = bytes;
-    base += align256(bytes);
-    left -= align256(bytes);
-  };
-  void *ws_cs, *ws_act, *ws_dw;
-  size_t n_cs, n_act, n_dw;
-  carve(need.colsum, &ws_cs, &n_cs);
-  carve(need.dw, &ws_dw, &n_dw);
-  carve(need.act, &ws_act, &n_act);
+  // Every launch gets the caller's buffer when it is large enough for that launch, and none
+  // otherwise (same results from the plain form of the launch).  Bias gradients cannot do without.
+  auto fits = [&](size_t bytes) { return workspace != nullptr && bytes > 0 && bytes <= workspace_bytes; };
+  void* const ws_cs = fits(need.colsum) ? workspace : nullptr;
+  void* const ws_dw = fits(need.dw) ? workspace : nullptr;
+  void* const ws_act = fits(need.act) ? workspace : nullptr;
+  const size_t n_dw = ws_dw ? workspace_bytes : 0, n_act = ws_act ? workspace_bytes : 0;
   if (need.colsum > 0 && ws_cs == nullptr)
     return fail(GMLP_EINVAL, "%s: bias gradients need a workspace of at least %zu bytes (gmlp_mlp_workspace_bytes)",
-                __func__, align256(need.colsum));
+                __func__, need.colsum);
 
   const void* lhs[3]; const void* rhs[3]; void* dws[3]; int64_t R[3], C[3];
   int n = 0;
