@@ -156,6 +156,21 @@ def test_whole_pass_entry_points_validate_before_touching_the_device():
     assert lib.gmlp_mlp_workspace_bytes(7, 8, 8, 8, 0) == 0 and lib.gmlp_mlp_workspace_bytes(0, 0, 8, 8, 0) == 0
 
 
+def test_activation_tables_of_the_reference_are_importable():
+    """ACT2CLS / ACT2FN / ClassInstantier (src/triton_gated_mlp/gated_mlp.py:10-26): name -> module
+    class, and a table whose lookup instantiates."""
+    from triton_gated_mlp.gated_mlp import ACT2CLS, ACT2FN, ClassInstantier
+
+    assert set(ACT2CLS) == {"gelu", "leaky_relu", "relu", "sigmoid", "silu", "swish", "tanh"}
+    assert ACT2CLS["swish"] is torch.nn.SiLU and ACT2CLS["gelu"] is torch.nn.GELU
+    a, b = ACT2FN["silu"], ACT2FN["silu"]
+    assert isinstance(a, torch.nn.SiLU) and a is not b
+    table = ClassInstantier({"leaky": (torch.nn.LeakyReLU, {"negative_slope": 0.2})})
+    assert table["leaky"].negative_slope == 0.2
+    with pytest.raises(KeyError):
+        ACT2FN["no_such_act"]
+
+
 def test_error_codes_map_to_python_exceptions():
     lib = _cabi.lib()
     _, a = _buf()

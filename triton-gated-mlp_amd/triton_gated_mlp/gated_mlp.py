@@ -26,6 +26,23 @@ from .ops import fwd as _fwd
 from .ops.bwd import mlp_hidden_states_bwd
 from .ops.fwd import mlp_hidden_states_fwd
 
+class _FreshModule(dict):
+    """Mapping name -> module class whose lookup hands out a NEW module instance (a value may be a
+    (class, kwargs) pair): the behaviour of the reference's ACT2FN table
+    (src/triton_gated_mlp/gated_mlp.py:10-26)."""
+
+    def __getitem__(self, key):
+        entry = super().__getitem__(key)
+        cls, kwargs = entry if isinstance(entry, tuple) else (entry, {})
+        return cls(**kwargs)
+
+
+ACT2CLS = {name: type(mod) for name, mod in (
+    ("gelu", nn.GELU()), ("leaky_relu", nn.LeakyReLU()), ("relu", nn.ReLU()), ("sigmoid", nn.Sigmoid()),
+    ("silu", nn.SiLU()), ("swish", nn.SiLU()), ("tanh", nn.Tanh()))}
+ACT2FN = _FreshModule(ACT2CLS)
+ClassInstantier = _FreshModule  # the reference's name for it
+
 ACT_FWD = {
     "gelu": nn.GELU(),
     "leaky_relu": nn.LeakyReLU(),
